@@ -73,10 +73,21 @@ class KVGroup:
 
     def bytes_per_token(self) -> int:
         return (len(self.entries) * self.request.kv_heads * (self.request.head_dim + self.request.value_head_dim)
-                * self.k.element_size())
+                * self.k.element_size()) // self.request.every
+
+    def entries_of(self, length: int) -> int:
+        """Entries that a sequence of ``length`` tokens holds here: one a token, or one for every whole block of
+        ``request.every`` tokens."""
+        return int(length) // self.request.every
+
+    def pages_needed(self, slot: int, new_length: int) -> int:
+        return self.table.pages_needed(slot, self.entries_of(new_length))
+
+    def shrink(self, slot: int, new_length: int) -> int:
+        return self.table.shrink(slot, self.entries_of(new_length))
 
     def grow(self, slot: int, new_length: int) -> None:
-        changed = self.table.grow(slot, new_length)
+        changed = self.table.grow(slot, self.entries_of(new_length))
         if changed:
             self._settle()
             row = self.table.rows[slot]
@@ -123,6 +134,7 @@ class SequenceCache:
         self.lengths: Dict[int, int] = {}
 
         self.kv_groups: List[KVGroup] = []
+        self._strides: Tuple[int, ...] = ()  # the groups' ``every`` beyond 1
         self.state_regions: Dict[str, torch.Tensor] = {}
         self._layer_state: List[str] = []  # regions that a mixer's StateRequest asked for
         self._views: Dict[int, Any] = {}
@@ -160,6 +172,8 @@ class SequenceCache:
             for position, place in enumerate(entries):
                 single[place] = KVView(group.k[position], group.v[position], group.block_table, request.window, False)
 
+        self._strides = tuple(sorted({group.request.every for group in self.kv_groups if group.request.every > 1}))
+
         def gather(index, path, request):
             if isinstance(request, (tuple, list)):
                 return tuple(gather(index, path + (position,), inner) for position, inner in enumerate(request))
@@ -181,7 +195,10 @@ class SequenceCache:
 
         for index, owner in shared.items():
             view = shared_view(self._views.get(owner))
-            if view is not None:
+            if index in self._views:
+                # an entry that reads another's cache and keeps something of its own beside it sees both
+                self._views[index] = (view, self._views[index])
+            elif view is not None:
                 self._views[index] = view
 
     # ---- state regions ----------------------------------------------------
@@ -235,7 +252,7 @@ class SequenceCache:
                 f"slot {slot}: a model that keeps fixed-size state per sequence ({', '.join(self._layer_state)}) cannot be "
                 "truncated; release the slot and run the tokens again")
         for group in self.kv_groups:
-            group.table.shrink(slot, int(length))
+            group.shrink(slot, int(length))
         self.lengths[slot] = int(length)
 
     def reset(self, slot: int) -> None:
@@ -247,7 +264,7 @@ class SequenceCache:
         on drawing where it was."""
         self.length(slot)  # raises if the slot is not held
         for group in self.kv_groups:
-            group.table.shrink(slot, 0)
+            group.shrink(slot, 0)
         self.lengths[slot] = 0
         for name in self._layer_state:
             self.state_regions[name][slot].zero_()
@@ -260,7 +277,7 @@ class SequenceCache:
         for slot, length in lengths.items():
             if slot in self.lengths and 0 <= int(length) < self.lengths[slot]:
                 for group in self.kv_groups:
-                    group.table.shrink(slot, int(length))
+                    group.shrink(slot, int(length))
                 self.lengths[slot] = int(length)
 
     def check_room(self, growth: Dict[int, int]) -> None:
@@ -277,7 +294,7 @@ class SequenceCache:
         for group in self.kv_groups:
             need = 0
             for slot, extra in growth.items():
-                need += group.table.pages_needed(slot, self.lengths[slot] + extra)
+                need += group.pages_needed(slot, self.lengths[slot] + extra)
             if need > group.table.pool.free:
                 raise CacheFull(
                     f"the cache has {group.table.pool.free} free pages of {PAGE_TOKENS} tokens; this step needs {need}"
@@ -301,7 +318,9 @@ class SequenceCache:
             before = [lengths[slot] for slot in slots]
         except KeyError as error:
             raise InvalidInput(f"cache slot {error.args[0]} is not held") from None
-        crossing = {slot: 1 for slot, length in zip(slots, before) if length % PAGE_TOKENS == 0}
+        # (a group that keeps one entry for every block of tokens starts a page where a block that opens one is completed)
+        crossing = {slot: 1 for slot, length in zip(slots, before) if length % PAGE_TOKENS == 0 or any(
+            (length + 1) % (PAGE_TOKENS * every) == every for every in self._strides)}
         if before and max(before) >= self.max_positions:
             self.check_room({slot: 1 for slot in slots})  # raises, naming the slot
         if crossing:

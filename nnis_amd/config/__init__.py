@@ -1,5 +1,7 @@
 from .llama import LlamaConfig, read_config_json  # noqa: F401
 from .zifunex import ZifunexConfig  # noqa: F401
+from .mutedra import MutedraConfig  # noqa: F401
+from .robopel import RobopelConfig  # noqa: F401
 from .presets import preset, preset_names  # noqa: F401
 from .registry import (  # noqa: F401
     Architecture,

@@ -78,6 +78,14 @@ struct AttnArgs {
   const float* bias;   // [heads, reach + 1]: added to the scaled score of a key `n` positions back, row min(n, reach)
   int reach;
   const float* sink;   // [heads]: a score that joins the softmax's denominator and has no value
+  // Pooled blocks beside a window (the row kernel only), off when `pool` is zero: entry b of a second set of pages
+  // stands for the positions b * pool .. b * pool + pool - 1 and is seen by a query at position p, in the same
+  // softmax as the window's keys, once the whole block has left the window: b * pool + pool - 1 <= p - window.
+  const void* pool_k;
+  const void* pool_v;
+  const int* pool_table;  // [slots][pool_max_pages]
+  int pool_max_pages;
+  int pool;
 };
 
 // One wave per (token, query head); lanes take keys lo+lane, lo+lane+64, ...,
@@ -118,7 +126,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
   for (int d = 0; d < HDV; ++d) o[d] = 0.0f;
   const float* bias_row = a.bias ? a.bias + (size_t)head * (a.reach + 1) : nullptr;
 
-  auto take = [&](int j) {
+  auto take = [&](const CacheT* kp, const CacheT* vp, const int* pages, int j, bool near) {
     const int page = pages[j / kPageTokens];
     const int r = j % kPageTokens;
     const CacheT* keys = kp + ((size_t)page * a.kv_heads + kv_head) * nnis_k_page_elems(HD);
@@ -127,7 +135,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
     for (int d = 0; d < HD; ++d) dot = fmaf(qs[d], to_f32(keys[nnis_k_offset(r, d)]), dot);
     float s = dot * a.scale;
     if (a.softcap > 0.0f) s = a.softcap * tanhf(s / a.softcap);
-    if (bias_row) s += bias_row[min(pos - j, a.reach)];
+    if (bias_row && near) s += bias_row[min(pos - j, a.reach)];
     const float m_new = fmaxf(m, s);
     const float alpha = expf(m - m_new);  // exp(-inf) = 0 on the first key
     const float p = expf(s - m_new);
@@ -138,8 +146,14 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
     m = m_new;
   };
   const int kept = min(a.keep_first, lo);  // the kept first keys that the window has left behind
-  for (int j = lane; j < kept; j += kWave) take(j);
-  for (int j = lo + lane; j < kv_len; j += kWave) take(j);
+  for (int j = lane; j < kept; j += kWave) take(kp, vp, pages, j, true);
+  for (int j = lo + lane; j < kv_len; j += kWave) take(kp, vp, pages, j, true);
+  if (a.pool > 0 && lo >= a.pool) {
+    // the blocks that lie wholly before the window: block b ends at b * pool + pool - 1 <= pos - window = lo - 1
+    const int* pool_pages = a.pool_table + (size_t)slot * a.pool_max_pages;
+    const int blocks = lo / a.pool;
+    for (int b = lane; b < blocks; b += kWave) take((const CacheT*)a.pool_k, (const CacheT*)a.pool_v, pool_pages, b, false);
+  }
 
   float m_all = wave_max(m);
   const float sink = a.sink ? a.sink[head] : -INFINITY;
@@ -1318,11 +1332,15 @@ __global__ void attention_combine_kernel(const float* __restrict__ partial, bf16
 
 }  // namespace
 
-extern "C" int nnis_attention_rows_more(const void* q, int q_dtype, void* out, int out_dtype, const void* k_pages,
-                                   const void* v_pages, int cache_dtype, const int* block_table, int max_pages,
-                                   const int* tok_slot, const int* tok_pos, int tokens, int heads, int kv_heads,
-                                   int head_dim, int window, float scale, int value_dim, float softcap, int keep_first,
-                                        const float* bias, int reach, const float* sink, void* stream) {
+extern "C" int nnis_attention_rows_pooled(const void* q, int q_dtype, void* out, int out_dtype, const void* k_pages,
+                                          const void* v_pages, int cache_dtype, const int* block_table, int max_pages,
+                                          const int* tok_slot, const int* tok_pos, int tokens, int heads, int kv_heads,
+                                          int head_dim, int window, float scale, int value_dim, float softcap, int keep_first,
+                                          const float* bias, int reach, const float* sink, const void* pool_k,
+                                          const void* pool_v, const int* pool_table, int pool_max_pages, int pool,
+                                          void* stream) {
+  NNIS_REQUIRE(pool >= 0 && (pool == 0 || (window > 0 && pool_k && pool_v && pool_table && pool_max_pages > 0)),
+               "attention: pooled blocks (%d tokens each) need a window and pages of their own", pool);
   NNIS_REQUIRE(head_dim == HD, "attention: this module is compiled for head_dim %d, got %d", HD, head_dim);
   NNIS_REQUIRE((value_dim <= 0 ? head_dim : value_dim) == HDV, "attention: this module is compiled for values of %d channels, got %d", HDV, value_dim);
   NNIS_REQUIRE(softcap >= 0.0f, "attention: the cap of the scores must not be negative, got %g", (double)softcap);
@@ -1339,6 +1357,7 @@ extern "C" int nnis_attention_rows_more(const void* q, int q_dtype, void* out, i
   a.block_table = block_table; a.max_pages = max_pages; a.tok_slot = tok_slot; a.tok_pos = tok_pos;
   a.tokens = tokens; a.heads = heads; a.kv_heads = kv_heads; a.window = window; a.scale = scale; a.softcap = softcap;
   a.keep_first = window > 0 ? keep_first : 0; a.bias = bias; a.reach = reach; a.sink = sink;
+  a.pool_k = pool_k; a.pool_v = pool_v; a.pool_table = pool_table; a.pool_max_pages = pool_max_pages; a.pool = pool;
   const long long items = (long long)tokens * heads;
   const unsigned blocks = (unsigned)((items + 3) / 4);
   if (cache_dtype == NNIS_F32) {
@@ -1350,6 +1369,16 @@ extern "C" int nnis_attention_rows_more(const void* q, int q_dtype, void* out, i
   return 0;
 }
 
+
+extern "C" int nnis_attention_rows_more(const void* q, int q_dtype, void* out, int out_dtype, const void* k_pages,
+                                        const void* v_pages, int cache_dtype, const int* block_table, int max_pages,
+                                        const int* tok_slot, const int* tok_pos, int tokens, int heads, int kv_heads,
+                                        int head_dim, int window, float scale, int value_dim, float softcap, int keep_first,
+                                        const float* bias, int reach, const float* sink, void* stream) {
+  return nnis_attention_rows_pooled(q, q_dtype, out, out_dtype, k_pages, v_pages, cache_dtype, block_table, max_pages, tok_slot,
+                                    tok_pos, tokens, heads, kv_heads, head_dim, window, scale, value_dim, softcap, keep_first,
+                                    bias, reach, sink, nullptr, nullptr, nullptr, 0, 0, stream);
+}
 
 extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int out_dtype, const void* k_pages,
                                    const void* v_pages, int cache_dtype, const int* block_table, int max_pages,

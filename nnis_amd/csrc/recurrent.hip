@@ -725,3 +725,114 @@ extern "C" int nnis_head_norm_gate(const float* o, const void* gate, int gate_dt
   NNIS_LAUNCH_CHECK("head_norm_gate");
   return 0;
 }
+
+// -----------------------------------------------------------------------------
+// minGRU: a gated recurrence whose gates read the current token only.  Per channel
+//     z = sigmoid(zp + bz),  u = up + bu,  c = u + 1/2 where u >= 0 and sigmoid(u) below,
+//     S <- (1 - z) S + z c,  out = S * silu(g)
+// over each sequence's rows, from and into state [slots, width] (32-bit).  `rows` is the fused projection's output
+// [tokens, stride]: zp in columns 0 .. width - 1, up in the next `width`, g in the next.  A thread a channel.  The
+// recurrence is linear in S, so a long run is cut into pieces (PASS 1: every piece but a sequence's last from a zero
+// state, leaving the product of its 1 - z and its end state; PASS 2: every piece again from the state that the
+// pieces before it hand on, which it adds up itself, writing the outputs, the last piece the sequence's state).
+// -----------------------------------------------------------------------------
+namespace {
+
+struct MinGruArgs {
+  const void* rows;
+  int dtype, stride;
+  const void* z_bias;
+  const void* x_bias;
+  int bias_dtype;
+  float* state;
+  const int* seq_slot;
+  const int* seq_start;
+  int batch, width;
+  void* out;
+  int out_dtype;
+  int piece, pieces;  // tokens of a piece, most pieces of a sequence; pieces == 1: not cut
+  float* decay;       // [batch, pieces, width]: a piece's product of 1 - z
+  float* ends;        // [batch, pieces, width]: a piece's end state from zero
+};
+
+template <int PASS>
+__global__ __launch_bounds__(256) void min_gru_kernel(MinGruArgs a) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int b = blockIdx.y / a.pieces;
+  const int piece = blockIdx.y % a.pieces;
+  const int slot = a.seq_slot[b];
+  if (slot < 0 || c >= a.width) return;
+  const int start = a.seq_start[b], stop = a.seq_start[b + 1];
+  int first = start, last = stop;
+  if (a.pieces > 1) {
+    first = start + piece * a.piece;
+    last = min(stop, first + a.piece);
+    if (first >= stop) return;
+    if (PASS == 1 && last == stop && piece > 0) return;  // a last piece's end state is the second pass's business (the first piece still keeps the state's copy)
+  }
+  const float bz = a.z_bias ? load_as_f32(a.z_bias, a.bias_dtype, c) : 0.0f;
+  const float bu = a.x_bias ? load_as_f32(a.x_bias, a.bias_dtype, c) : 0.0f;
+  float s = 0.0f, keep = 1.0f;
+  const size_t mine = ((size_t)b * a.pieces + piece) * a.width + c;
+  if (a.pieces == 1) {
+    s = a.state[(size_t)slot * a.width + c];
+  } else if (PASS == 1) {
+    // the first piece runs from the sequence's state and keeps a copy of it where its product would go: the second
+    // pass reads no state (its last piece writes it while others may not have started)
+    if (piece == 0) a.decay[mine] = s = a.state[(size_t)slot * a.width + c];
+  } else if (piece == 0) {
+    s = a.decay[mine];
+  } else {
+    // what the pieces before this one hand on: the first piece's end, then I <- decay_k I + ends_k piece by piece
+    s = a.ends[(size_t)b * a.pieces * a.width + c];
+    for (int k = 1; k < piece; ++k) {
+      const size_t at = ((size_t)b * a.pieces + k) * a.width + c;
+      s = fmaf(a.decay[at], s, a.ends[at]);
+    }
+  }
+  for (int t = first; t < last; ++t) {
+    const size_t at = (size_t)t * a.stride + c;
+    const float z = sigmoid_f(load_as_f32(a.rows, a.dtype, at) + bz);
+    const float u = load_as_f32(a.rows, a.dtype, at + a.width) + bu;
+    const float cand = u >= 0.0f ? u + 0.5f : sigmoid_f(u);
+    s = fmaf(z, cand - s, s);  // (1 - z) s + z cand
+    if (PASS == 1) {
+      keep *= 1.0f - z;
+    } else {
+      const float g = load_as_f32(a.rows, a.dtype, at + 2 * (size_t)a.width);
+      store_from_f32(a.out, a.out_dtype, (size_t)t * a.width + c, s * g * sigmoid_f(g));
+    }
+  }
+  if (PASS == 1) {
+    if (piece > 0) a.decay[mine] = keep;
+    a.ends[mine] = s;
+  } else if (last == stop) {
+    a.state[(size_t)slot * a.width + c] = s;
+  }
+}
+
+}  // namespace
+
+extern "C" int nnis_min_gru(const void* rows, int dtype, int stride, const void* z_bias, const void* x_bias, int bias_dtype, float* state,
+                            const int* seq_slot, const int* seq_start, int batch, int width, void* out, int out_dtype, int piece,
+                            int pieces, float* decay, float* ends, void* stream) {
+  NNIS_REQUIRE(rows && state && seq_slot && seq_start && out, "min_gru: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(dtype) && nnis_dtype_ok(out_dtype) && ((z_bias == nullptr && x_bias == nullptr) || nnis_dtype_ok(bias_dtype)),
+               "min_gru: unknown dtype");
+  NNIS_REQUIRE(width > 0 && stride >= 3 * width, "min_gru: rows of %d columns do not hold three times %d channels", stride, width);
+  NNIS_REQUIRE(pieces >= 1 && (pieces == 1 || (piece > 0 && decay && ends)), "min_gru: pieces without scratch");
+  if (batch <= 0) return 0;
+  MinGruArgs a;
+  a.rows = rows; a.dtype = dtype; a.stride = stride; a.z_bias = z_bias; a.x_bias = x_bias; a.bias_dtype = bias_dtype;
+  a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.batch = batch; a.width = width; a.out = out;
+  a.out_dtype = out_dtype; a.piece = piece; a.pieces = pieces; a.decay = decay; a.ends = ends;
+  const int threads = width >= 256 ? 256 : 64;
+  const dim3 grid((width + threads - 1) / threads, batch * pieces);
+  if (pieces > 1) {
+    hipLaunchKernelGGL(min_gru_kernel<1>, grid, dim3(threads), 0, (hipStream_t)stream, a);
+    NNIS_LAUNCH_CHECK("min_gru (first pass)");
+  }
+  hipLaunchKernelGGL(min_gru_kernel<2>, grid, dim3(threads), 0, (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("min_gru");
+  return 0;
+}

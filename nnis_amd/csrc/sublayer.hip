@@ -1,0 +1,464 @@
+// What lies between the projections of sublayers that norm their outputs, gate their heads, pool their keys or
+// route their tokens: row-wise kernels, all 32-bit inside whatever the storage type.
+//
+//   cast_rows          rows of one type as rows of another (the 32-bit stream as a sublayer's input)
+//   rms_post_step      x += y / rms(y) * (offset + w), and the stream's rows in the activation type
+//   poly_norm          a N(z) + b N(z^2) + c N(z^3) + e, N a division by the root mean square of a row
+//   route_top          softmax of router logits, the `top` largest of score + correction, dense weights out
+//   routed_act         weight[row, expert] * relu(z)^2 on the experts' fused up projection
+//   rows_axpy          y[row] += c[row] * h[row]
+//   sigmoid_gate       o *= sigmoid(g)
+//   head_norm_write    per-head RMS norm of queries and keys, rotation (neighbouring channels or halves), queries out,
+//                      keys and values into the pages
+//   pool_blocks        the mean key and value of every block of `pool` tokens that a step completes
+#include "common.h"
+
+thread_local char g_nnis_error[512] = {0};
+extern "C" const char* nnis_last_error() { return g_nnis_error; }
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// -----------------------------------------------------------------------------
+// The way out of a sublayer whose output alone is normed: x[row] += y[row] / sqrt(mean(y^2) + eps) * (offset + w),
+// in place in the 32-bit stream, and h[row] = the new x in the activation type (what the next sublayer reads).
+// A block a row; the row is read twice (the second time from the caches).
+// -----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rms_post_step_kernel(float* __restrict__ x, const void* __restrict__ y, int y_dtype,
+                                                            const void* __restrict__ weight, int w_dtype, float offset, float eps,
+                                                            void* __restrict__ h, int h_dtype, int width) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * width;
+  float ss = 0.0f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = load_as_f32(y, y_dtype, base + c);
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = load_as_f32(y, y_dtype, base + c);
+    const float sum = x[base + c] + v * inv * (offset + load_as_f32(weight, w_dtype, c));
+    x[base + c] = sum;
+    if (h) store_from_f32(h, h_dtype, base + c, sum);
+  }
+}
+
+// -----------------------------------------------------------------------------
+// PolyNorm: out = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e, powers element by element, each root mean
+// square over the row with eps inside the root; coef = (a, b, c, e) in device memory.
+// -----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void poly_norm_kernel(const void* __restrict__ z, int z_dtype, const float* __restrict__ coef,
+                                                        float eps, void* __restrict__ out, int out_dtype, int width) {
+  __shared__ float scratch[3][16];
+  const size_t base = (size_t)blockIdx.x * width;
+  float s2 = 0.0f, s4 = 0.0f, s6 = 0.0f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = load_as_f32(z, z_dtype, base + c);
+    const float v2 = v * v;
+    s2 += v2;
+    s4 = fmaf(v2, v2, s4);
+    s6 = fmaf(v2 * v, v2 * v, s6);
+  }
+  const float n = (float)width;
+  const float i1 = 1.0f / sqrtf(block_sum(s2, scratch[0]) / n + eps);
+  const float i2 = 1.0f / sqrtf(block_sum(s4, scratch[1]) / n + eps);
+  const float i3 = 1.0f / sqrtf(block_sum(s6, scratch[2]) / n + eps);
+  const float a = coef[0] * i1, b = coef[1] * i2, cc = coef[2] * i3, e = coef[3];
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = load_as_f32(z, z_dtype, base + c);
+    store_from_f32(out, out_dtype, base + c, fmaf(v, fmaf(v, fmaf(v, cc, b), a), e));
+  }
+}
+
+// -----------------------------------------------------------------------------
+// Routing: scores s = softmax(logits) over n outputs; the `top` outputs with the largest s + correction are chosen
+// (the lower index on a tie); gates[row, e] = s_e for a chosen output below `experts`, 0 for the others; keep[row] =
+// the sum of s over the chosen outputs from `experts` on (those hand the input through).  A wave a row.
+// -----------------------------------------------------------------------------
+constexpr int kRouteMost = 16;  // outputs a lane holds: n <= 64 * kRouteMost
+
+__global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int rows,
+                                                        int n, int experts, int top, float* __restrict__ gates,
+                                                        float* __restrict__ keep) {
+  const int row = blockIdx.x * 4 + threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  if (row >= rows) return;
+  float s[kRouteMost], choice[kRouteMost];
+  float top_logit = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < kRouteMost; ++i) {
+    const int e = i * kWave + lane;
+    s[i] = e < n ? logits[(size_t)row * n + e] : -INFINITY;
+    top_logit = fmaxf(top_logit, s[i]);
+  }
+  top_logit = wave_max(top_logit);
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kRouteMost; ++i) {
+    s[i] = (i * kWave + lane) < n ? expf(s[i] - top_logit) : 0.0f;
+    sum += s[i];
+  }
+  const float inv = 1.0f / wave_sum(sum);
+  unsigned chosen = 0;
+#pragma unroll
+  for (int i = 0; i < kRouteMost; ++i) {
+    const int e = i * kWave + lane;
+    s[i] *= inv;
+    choice[i] = e < n ? s[i] + (correction ? correction[e] : 0.0f) : -INFINITY;
+  }
+  float kept = 0.0f;
+  for (int round = 0; round < top; ++round) {
+    float best = -INFINITY;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < kRouteMost; ++i) {
+      const int e = i * kWave + lane;
+      if (!(chosen >> i & 1u) && e < n && (choice[i] > best || (choice[i] == best && e < best_e))) {
+        best = choice[i];
+        best_e = e;
+      }
+    }
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+      const float other = __shfl_xor(best, offset, kWave);
+      const int other_e = __shfl_xor(best_e, offset, kWave);
+      if (other > best || (other == best && other_e < best_e)) {
+        best = other;
+        best_e = other_e;
+      }
+    }
+    if (best_e == 0x7fffffff) break;  // fewer outputs than `top`
+    if (best_e % kWave == lane) {
+      const int i = best_e / kWave;
+      chosen |= 1u << i;
+#pragma unroll
+      for (int k = 0; k < kRouteMost; ++k)
+        if (k == i && best_e >= experts) kept += s[k];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kRouteMost; ++i) {
+    const int e = i * kWave + lane;
+    if (e < experts) gates[(size_t)row * experts + e] = (chosen >> i & 1u) ? s[i] : 0.0f;
+  }
+  kept = wave_sum(kept);
+  if (lane == 0) keep[row] = kept;
+}
+
+// out[row, e * ff + c] = gates[row, e] * relu(z[row, e * ff + c])^2
+__global__ void routed_act_kernel(const void* __restrict__ z, int z_dtype, const float* __restrict__ gates, void* __restrict__ out,
+                                  int out_dtype, int experts, int ff, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t per_row = (size_t)experts * ff;
+  const size_t row = i / per_row;
+  const int e = (int)((i % per_row) / ff);
+  const float g = gates[row * experts + e];
+  const float v = fmaxf(load_as_f32(z, z_dtype, i), 0.0f);
+  store_from_f32(out, out_dtype, i, g == 0.0f ? 0.0f : g * v * v);
+}
+
+// y[row, c] += keep[row] * h[row, c]
+__global__ void rows_axpy_kernel(void* __restrict__ y, int y_dtype, const void* __restrict__ h, int h_dtype,
+                                 const float* __restrict__ keep, int width, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const float k = keep[i / width];
+  if (k != 0.0f) store_from_f32(y, y_dtype, i, fmaf(k, load_as_f32(h, h_dtype, i), load_as_f32(y, y_dtype, i)));
+}
+
+// o[row, c] *= sigmoid(g[row * g_stride + c])
+__global__ void sigmoid_gate_kernel(void* __restrict__ o, int o_dtype, const void* __restrict__ g, int g_dtype, int g_stride,
+                                    int width, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t row = i / width;
+  const int c = (int)(i % width);
+  store_from_f32(o, o_dtype, i, load_as_f32(o, o_dtype, i) * sigmoid_f(load_as_f32(g, g_dtype, row * g_stride + c)));
+}
+
+// -----------------------------------------------------------------------------
+// Queries and keys of a fused projection's rows, head by head: an RMS norm over the head's channels with a weight
+// shared by the heads (or none), then the rotation of the first rot_dim channels by the token's position -- channel
+// 2i with 2i + 1 (`neighbours`) or channel i with i + rot_dim / 2 --, pair i by the angle whose cosine and sine are
+// table[pos][i].  Queries go to q_out [tokens, heads * head_dim]; keys and the values beside them into the pages of
+// the token's slot.  A wave a (token, head); a key head's wave also copies its value head.
+// -----------------------------------------------------------------------------
+constexpr int kHeadMost = 1024;
+
+struct HeadWriteArgs {
+  const void* rows;  // [tokens, stride]
+  int dtype, stride;
+  int q_col, k_col, v_col;  // first columns of the queries, keys and values in a row; k_col < 0: no keys or values
+  void* q_out;
+  int q_dtype;
+  const void* q_weight;  // [head_dim] or null
+  const void* k_weight;
+  int w_dtype;
+  float eps;
+  const float* cos_table;  // [positions][rot_dim / 2] or null
+  const float* sin_table;
+  int table_positions, rot_dim, neighbours;
+  const int* tok_slot;
+  const int* tok_pos;
+  void* k_pages;
+  void* v_pages;
+  int cache_dtype;
+  const int* block_table;
+  int max_pages;
+  int heads, kv_heads, head_dim, value_dim;
+};
+
+__global__ __launch_bounds__(64) void head_norm_write_kernel(HeadWriteArgs a) {
+  __shared__ float row[kHeadMost];
+  const int token = blockIdx.x;
+  const int head = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int slot = a.tok_slot[token];
+  if (slot < 0) return;
+  const int pos = a.tok_pos[token];
+  const bool is_key = head >= a.heads;
+  const int hd = a.head_dim;
+  const size_t in = (size_t)token * a.stride + (is_key ? a.k_col + (head - a.heads) * hd : a.q_col + head * hd);
+  const void* weight = is_key ? a.k_weight : a.q_weight;
+  float ss = 0.0f;
+  for (int d = lane; d < hd; d += kWave) {
+    const float v = load_as_f32(a.rows, a.dtype, in + d);
+    row[d] = v;
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  __syncthreads();
+  if (weight) {
+    const float inv = 1.0f / sqrtf(ss / (float)hd + a.eps);
+    for (int d = lane; d < hd; d += kWave) row[d] = row[d] * inv * load_as_f32(weight, a.w_dtype, d);
+    __syncthreads();
+  }
+  const bool rotate = a.cos_table != nullptr && pos < a.table_positions;
+  const int half = a.rot_dim / 2;
+  int page = -1;
+  if (is_key) page = a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens];
+  const int in_page = pos % kPageTokens;
+  for (int d = lane; d < hd; d += kWave) {
+    float v = row[d];
+    if (rotate && d < a.rot_dim) {
+      int pair, partner;
+      bool first;
+      if (a.neighbours) {
+        pair = d / 2, first = (d % 2) == 0, partner = first ? d + 1 : d - 1;
+      } else {
+        first = d < half, pair = first ? d : d - half, partner = first ? d + half : d - half;
+      }
+      const float c = a.cos_table[(size_t)pos * half + pair], s = a.sin_table[(size_t)pos * half + pair];
+      v = first ? v * c - row[partner] * s : v * c + row[partner] * s;
+    }
+    if (!is_key) {
+      store_from_f32(a.q_out, a.q_dtype, ((size_t)token * a.heads + head) * hd + d, v);
+    } else {
+      const size_t dst = ((size_t)page * a.kv_heads + (head - a.heads)) * nnis_k_page_elems(hd);
+      store_from_f32(a.k_pages, a.cache_dtype, dst + nnis_k_offset(in_page, d), v);
+    }
+  }
+  if (is_key) {
+    const int kv_head = head - a.heads;
+    const int vd = a.value_dim;
+    const size_t src = (size_t)token * a.stride + a.v_col + (size_t)kv_head * vd;
+    const size_t dst = ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(vd);
+    for (int d = lane; d < vd; d += kWave)
+      store_from_f32(a.v_pages, a.cache_dtype, dst + nnis_v_offset(d, in_page), load_as_f32(a.rows, a.dtype, src + d));
+  }
+}
+
+// -----------------------------------------------------------------------------
+// Pooled blocks: a token at position p with (p + 1) % pool == 0 completes block b = p / pool of its sequence; the
+// block's key is the mean of its `pool` keys as the pages hold them, its value the mean of their values; both go to
+// entry b of a second set of pages with a block table of its own.  Runs behind the step's cache write.
+// -----------------------------------------------------------------------------
+struct PoolArgs {
+  const void* k_pages;
+  const void* v_pages;
+  int cache_dtype;
+  const int* block_table;
+  int max_pages;
+  void* pool_k;
+  void* pool_v;
+  const int* pool_table;
+  int pool_max_pages;
+  const int* tok_slot;
+  const int* tok_pos;
+  int kv_heads, head_dim, value_dim, pool;
+};
+
+__global__ __launch_bounds__(128) void pool_blocks_kernel(PoolArgs a) {
+  const int token = blockIdx.x;
+  const int kv_head = blockIdx.y;
+  const int slot = a.tok_slot[token];
+  if (slot < 0) return;
+  const int pos = a.tok_pos[token];
+  if ((pos + 1) % a.pool != 0) return;
+  const int b = pos / a.pool;
+  const int first = b * a.pool;
+  const int* pages = a.block_table + (size_t)slot * a.max_pages;
+  const int out_page = a.pool_table[(size_t)slot * a.pool_max_pages + b / kPageTokens];
+  const int out_at = b % kPageTokens;
+  const float share = 1.0f / (float)a.pool;
+  const int hd = a.head_dim, vd = a.value_dim;
+  for (int d = threadIdx.x; d < hd + vd; d += blockDim.x) {
+    const bool key = d < hd;
+    const int c = key ? d : d - hd;
+    float sum = 0.0f;
+    for (int j = 0; j < a.pool; ++j) {
+      const int p = first + j;
+      const size_t page = (size_t)pages[p / kPageTokens] * a.kv_heads + kv_head;
+      sum += key ? load_as_f32(a.k_pages, a.cache_dtype, page * nnis_k_page_elems(hd) + nnis_k_offset(p % kPageTokens, c))
+                 : load_as_f32(a.v_pages, a.cache_dtype, page * nnis_v_page_elems(vd) + nnis_v_offset(c, p % kPageTokens));
+    }
+    const size_t out = (size_t)out_page * a.kv_heads + kv_head;
+    if (key) {
+      store_from_f32(a.pool_k, a.cache_dtype, out * nnis_k_page_elems(hd) + nnis_k_offset(out_at, c), sum * share);
+    } else {
+      store_from_f32(a.pool_v, a.cache_dtype, out * nnis_v_page_elems(vd) + nnis_v_offset(c, out_at), sum * share);
+    }
+  }
+}
+
+// out[r, :] = x[rows ? rows[r] : r, :] in the output's type
+__global__ void cast_rows_kernel(const void* __restrict__ x, int x_dtype, void* __restrict__ out, int out_dtype,
+                                 const int* __restrict__ rows, int width, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t r = i / width;
+  const size_t from = rows ? (size_t)rows[r] * width + i % width : i;
+  store_from_f32(out, out_dtype, i, load_as_f32(x, x_dtype, from));
+}
+
+inline unsigned blocks_for(size_t total, int threads) { return (unsigned)((total + threads - 1) / threads); }
+
+}  // namespace
+
+extern "C" int nnis_cast_rows(const void* x, int x_dtype, void* out, int out_dtype, const int* rows, int out_rows, int width, void* stream) {
+  NNIS_REQUIRE(x && out && width > 0, "cast_rows: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(x_dtype) && nnis_dtype_ok(out_dtype), "cast_rows: unknown dtype");
+  if (out_rows <= 0) return 0;
+  const size_t total = (size_t)out_rows * width;
+  hipLaunchKernelGGL(cast_rows_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, (hipStream_t)stream, x, x_dtype, out, out_dtype, rows,
+                     width, total);
+  NNIS_LAUNCH_CHECK("cast_rows");
+  return 0;
+}
+
+extern "C" int nnis_rms_post_step(float* x, const void* y, int y_dtype, const void* weight, int w_dtype, float offset, float eps,
+                                  void* h, int h_dtype, int rows, int width, void* stream) {
+  NNIS_REQUIRE(x && y && weight && width > 0, "rms_post_step: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(w_dtype) && (h == nullptr || nnis_dtype_ok(h_dtype)), "rms_post_step: unknown dtype");
+  if (rows <= 0) return 0;
+  hipLaunchKernelGGL(rms_post_step_kernel, dim3(rows), dim3(width >= 1024 ? 256 : (width >= 256 ? 128 : 64)), 0, (hipStream_t)stream, x, y,
+                     y_dtype, weight, w_dtype, offset, eps, h, h_dtype, width);
+  NNIS_LAUNCH_CHECK("rms_post_step");
+  return 0;
+}
+
+extern "C" int nnis_poly_norm(const void* z, int z_dtype, const float* coef, float eps, void* out, int out_dtype, int rows, int width,
+                              void* stream) {
+  NNIS_REQUIRE(z && coef && out && width > 0, "poly_norm: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(z_dtype) && nnis_dtype_ok(out_dtype), "poly_norm: unknown dtype");
+  if (rows <= 0) return 0;
+  hipLaunchKernelGGL(poly_norm_kernel, dim3(rows), dim3(width >= 1024 ? 256 : (width >= 256 ? 128 : 64)), 0, (hipStream_t)stream, z, z_dtype,
+                     coef, eps, out, out_dtype, width);
+  NNIS_LAUNCH_CHECK("poly_norm");
+  return 0;
+}
+
+extern "C" int nnis_route_top(const float* logits, const float* correction, int rows, int n, int experts, int top, float* gates,
+                              float* keep, void* stream) {
+  NNIS_REQUIRE(logits && gates && keep, "route_top: missing operand");
+  NNIS_REQUIRE(n > 0 && n <= kWave * kRouteMost, "route_top: 1 to %d router outputs, got %d", kWave * kRouteMost, n);
+  NNIS_REQUIRE(experts >= 0 && experts <= n && top > 0 && top <= n, "route_top: %d experts and the %d largest of %d outputs", experts, top, n);
+  if (rows <= 0) return 0;
+  hipLaunchKernelGGL(route_top_kernel, dim3((rows + 3) / 4), dim3(256), 0, (hipStream_t)stream, logits, correction, rows, n, experts, top,
+                     gates, keep);
+  NNIS_LAUNCH_CHECK("route_top");
+  return 0;
+}
+
+extern "C" int nnis_routed_act(const void* z, int z_dtype, const float* gates, void* out, int out_dtype, int rows, int experts, int ff,
+                               void* stream) {
+  NNIS_REQUIRE(z && gates && out && experts > 0 && ff > 0, "routed_act: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(z_dtype) && nnis_dtype_ok(out_dtype), "routed_act: unknown dtype");
+  if (rows <= 0) return 0;
+  const size_t total = (size_t)rows * experts * ff;
+  hipLaunchKernelGGL(routed_act_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, (hipStream_t)stream, z, z_dtype, gates, out, out_dtype,
+                     experts, ff, total);
+  NNIS_LAUNCH_CHECK("routed_act");
+  return 0;
+}
+
+extern "C" int nnis_rows_axpy(void* y, int y_dtype, const void* h, int h_dtype, const float* keep, int rows, int width, void* stream) {
+  NNIS_REQUIRE(y && h && keep && width > 0, "rows_axpy: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(h_dtype), "rows_axpy: unknown dtype");
+  if (rows <= 0) return 0;
+  const size_t total = (size_t)rows * width;
+  hipLaunchKernelGGL(rows_axpy_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, (hipStream_t)stream, y, y_dtype, h, h_dtype, keep, width,
+                     total);
+  NNIS_LAUNCH_CHECK("rows_axpy");
+  return 0;
+}
+
+extern "C" int nnis_sigmoid_gate(void* o, int o_dtype, const void* g, int g_dtype, int g_stride, int rows, int width, void* stream) {
+  NNIS_REQUIRE(o && g && width > 0 && g_stride >= width, "sigmoid_gate: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(o_dtype) && nnis_dtype_ok(g_dtype), "sigmoid_gate: unknown dtype");
+  if (rows <= 0) return 0;
+  const size_t total = (size_t)rows * width;
+  hipLaunchKernelGGL(sigmoid_gate_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, (hipStream_t)stream, o, o_dtype, g, g_dtype, g_stride,
+                     width, total);
+  NNIS_LAUNCH_CHECK("sigmoid_gate");
+  return 0;
+}
+
+extern "C" int nnis_head_norm_write(const void* rows, int dtype, int stride, int q_col, int k_col, int v_col, void* q_out, int q_dtype,
+                                    const void* q_weight, const void* k_weight, int w_dtype, float eps, const float* cos_table,
+                                    const float* sin_table, int table_positions, int rot_dim, int neighbours, const int* tok_slot,
+                                    const int* tok_pos, void* k_pages, void* v_pages, int cache_dtype, const int* block_table,
+                                    int max_pages, int tokens, int heads, int kv_heads, int head_dim, int value_dim, void* stream) {
+  NNIS_REQUIRE(rows && q_out && tok_slot && tok_pos, "head_norm_write: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(dtype) && nnis_dtype_ok(q_dtype), "head_norm_write: unknown dtype");
+  NNIS_REQUIRE(heads > 0 && kv_heads >= 0 && head_dim > 0 && head_dim <= kHeadMost, "head_norm_write: heads of 1 to %d channels, got %d",
+               kHeadMost, head_dim);
+  NNIS_REQUIRE(rot_dim >= 0 && rot_dim <= head_dim && rot_dim % 2 == 0, "head_norm_write: rot_dim %d must be even and at most head_dim %d",
+               rot_dim, head_dim);
+  NNIS_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "head_norm_write: cos and sin tables must come together");
+  NNIS_REQUIRE((q_weight == nullptr && k_weight == nullptr) || nnis_dtype_ok(w_dtype), "head_norm_write: unknown weight dtype");
+  if (kv_heads > 0) {
+    NNIS_REQUIRE(k_col >= 0 && v_col >= 0 && k_pages && v_pages && block_table && max_pages > 0 && nnis_dtype_ok(cache_dtype) && value_dim > 0,
+                 "head_norm_write: keys without pages to go to");
+  }
+  if (tokens <= 0) return 0;
+  HeadWriteArgs a;
+  a.rows = rows; a.dtype = dtype; a.stride = stride; a.q_col = q_col; a.k_col = k_col; a.v_col = v_col;
+  a.q_out = q_out; a.q_dtype = q_dtype; a.q_weight = q_weight; a.k_weight = k_weight; a.w_dtype = w_dtype; a.eps = eps;
+  a.cos_table = cos_table; a.sin_table = sin_table; a.table_positions = table_positions; a.rot_dim = cos_table ? rot_dim : 0;
+  a.neighbours = neighbours; a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.k_pages = k_pages; a.v_pages = v_pages;
+  a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
+  a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim; a.value_dim = value_dim;
+  hipLaunchKernelGGL(head_norm_write_kernel, dim3(tokens, heads + kv_heads), dim3(64), 0, (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("head_norm_write");
+  return 0;
+}
+
+extern "C" int nnis_pool_blocks(const void* k_pages, const void* v_pages, int cache_dtype, const int* block_table, int max_pages,
+                                void* pool_k, void* pool_v, const int* pool_table, int pool_max_pages, const int* tok_slot,
+                                const int* tok_pos, int tokens, int kv_heads, int head_dim, int value_dim, int pool, void* stream) {
+  NNIS_REQUIRE(k_pages && v_pages && block_table && pool_k && pool_v && pool_table && tok_slot && tok_pos, "pool_blocks: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(cache_dtype) && max_pages > 0 && pool_max_pages > 0, "pool_blocks: bad pages");
+  NNIS_REQUIRE(kv_heads > 0 && head_dim > 0 && value_dim > 0 && pool > 0, "pool_blocks: bad sizes");
+  if (tokens <= 0) return 0;
+  PoolArgs a;
+  a.k_pages = k_pages; a.v_pages = v_pages; a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
+  a.pool_k = pool_k; a.pool_v = pool_v; a.pool_table = pool_table; a.pool_max_pages = pool_max_pages;
+  a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.kv_heads = kv_heads; a.head_dim = head_dim; a.value_dim = value_dim; a.pool = pool;
+  hipLaunchKernelGGL(pool_blocks_kernel, dim3(tokens, kv_heads), dim3(128), 0, (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("pool_blocks");
+  return 0;
+}

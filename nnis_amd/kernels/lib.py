@@ -55,7 +55,9 @@ PREBUILT_WIDE_VALUES = ("attn_hd7v5c", "attn_hd32v16c", "attn_hd16v48c", "attn_h
                         # with the scores' extras (kept first keys, bias by distance, sink), and latents as the one key/value head
                         "attn_hd32v16x", "attn_hd16v48x", "attn_hd48v32x", "attn_hd96v64x", "attn_hd32v24x", "attn_hd40", "attn_hd288v272x", "attn_hd16x",
                         # the sizes of the measurements of windowed and latent attention
-                        "attn_hd64x", "attn_hd128x", "attn_hd160v128x", "attn_hd256v192x")
+                        "attn_hd64x", "attn_hd128x", "attn_hd160v128x", "attn_hd256v192x",
+                        # capped scores with a sink: windows with pooled blocks
+                        "attn_hd16cx", "attn_hd32v16cx", "attn_hd24v40cx", "attn_hd64cx", "attn_hd128cx")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -137,6 +139,8 @@ register_module_family("attn_hd", _attention_recipe)
 register_module("recurrent", ["recurrent.hip"], headers=["common.h"])
 # attention over a cached latent: what lies between its projections (norms of the latents, rotation, cache write, gates)
 register_module("latent", ["latent.hip"], headers=["common.h"])
+# what lies between the projections of sublayers that norm their outputs, gate or pool their heads, or route their tokens
+register_module("sublayer", ["sublayer.hip"], headers=["common.h"])
 # plain host references of the kernels' operations, for the tests (no device code: the host compiler builds them)
 register_module("reference", ["reference.cpp"], host_only=True)
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-ffp-contract=off"]  # a multiply-add is fused only where the source says fmaf
@@ -310,7 +314,7 @@ def load_module(module: str, build_if_missing: bool = True) -> ctypes.CDLL:
 
 
 def all_prebuilt_modules() -> List[str]:
-    return ["core", "reference", "recurrent", "latent"] + [f"attn_hd{d}" for d in PREBUILT_HEAD_DIMS] + list(PREBUILT_WIDE_VALUES)
+    return ["core", "reference", "recurrent", "latent", "sublayer"] + [f"attn_hd{d}" for d in PREBUILT_HEAD_DIMS] + list(PREBUILT_WIDE_VALUES)
 
 
 def build_all(force: bool = True, jobs: int = 4) -> List[str]:

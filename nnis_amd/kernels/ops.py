@@ -68,6 +68,8 @@ _ATTN_SIGNATURES = {
                             _INT, _INT, _FLT, _INT, _FLT, _VOID],
     "nnis_attention_rows_more": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
                                  _INT, _INT, _FLT, _INT, _FLT, _INT, _VOID, _INT, _VOID, _VOID],
+    "nnis_attention_rows_pooled": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
+                                   _INT, _INT, _FLT, _INT, _FLT, _INT, _VOID, _INT, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _VOID],
     "nnis_attention_prefill_tile_rows": [_INT, _INT, _INT],
     "nnis_attention_prefill_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
                                     _INT, _INT, _INT, _FLT, _INT, _INT, _FLT, _VOID],
@@ -91,6 +93,20 @@ _RECURRENT_SIGNATURES = {
                       _VOID, _INT, _INT, _VOID, _VOID, _VOID],
     "nnis_gla_decays": [_VOID, _VOID, _INT, _INT, _FLT, _VOID],
     "nnis_head_norm_gate": [_VOID, _VOID, _INT, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _FLT, _VOID],
+    "nnis_min_gru": [_VOID, _INT, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT, _INT, _VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID],
+}
+
+_SUBLAYER_SIGNATURES = {
+    "nnis_cast_rows": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _VOID],
+    "nnis_rms_post_step": [_VOID, _VOID, _INT, _VOID, _INT, _FLT, _FLT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_poly_norm": [_VOID, _INT, _VOID, _FLT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_route_top": [_VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID],
+    "nnis_routed_act": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_rows_axpy": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _VOID],
+    "nnis_sigmoid_gate": [_VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_head_norm_write": [_VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID, _VOID, _INT, _FLT, _VOID, _VOID, _INT, _INT, _INT,
+                             _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_pool_blocks": [_VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
 }
 
 _LATENT_SIGNATURES = {
@@ -168,6 +184,18 @@ def latent():
     if _latent is None:
         _latent = _bind("latent", _LATENT_SIGNATURES)
     return _latent
+
+
+_sublayer = None
+
+
+def sublayer():
+    """The module of what lies between the projections of sublayers that norm their outputs, gate or pool their
+    heads, or route their tokens."""
+    global _sublayer
+    if _sublayer is None:
+        _sublayer = _bind("sublayer", _SUBLAYER_SIGNATURES)
+    return _sublayer
 
 
 def core():
@@ -494,14 +522,37 @@ class ScoreExtras:
             raise KernelError(f"attention: keep_first must not be negative, got {self.keep_first}")
 
 
+class PooledBlocks:
+    """Beside a window of ``window`` tokens: pages whose entry b holds one key
+    and one value for the tokens b * pool .. b * pool + pool - 1 of a
+    sequence (their means), with a block table of their own.  A query at
+    position p sees entry b once the whole block has left its window, b * pool
+    + pool - 1 <= p - window, in the same softmax as the window's keys."""
+
+    def __init__(self, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor, pool: int):
+        self.k_pages, self.v_pages, self.block_table, self.pool = k_pages, v_pages, block_table, int(pool)
+
+    def check(self, k_pages, v_pages, kv_heads: int, head_dim: int, value_dim: int, window: int) -> None:
+        _dev(self.k_pages, "pooled k_pages"), _dev(self.v_pages, "pooled v_pages"), _dev(self.block_table, "pooled block_table")
+        if self.pool <= 0 or not window:
+            raise KernelError(f"attention: pooled blocks of {self.pool} tokens beside a window of {window}")
+        if not _pages_fit(self.k_pages, self.v_pages, kv_heads, head_dim, value_dim) or self.k_pages.dtype != k_pages.dtype \
+                or self.v_pages.dtype != v_pages.dtype:
+            raise KernelError(f"attention: pooled page shapes {tuple(self.k_pages.shape)} / {tuple(self.v_pages.shape)} do not fit the keys'")
+        if self.block_table.dtype != torch.int32 or self.block_table.dim() != 2:
+            raise KernelError("attention: the pooled block_table must be int32 [slots, pages]")
+
+
 def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                    block_table: torch.Tensor, tok_slot: torch.Tensor, tok_pos: torch.Tensor, heads: int, kv_heads: int,
                    head_dim: int, scale: float, window: int = 0, value_dim: Optional[int] = None,
-                   softcap: float = 0.0, extras: Optional[ScoreExtras] = None) -> torch.Tensor:
+                   softcap: float = 0.0, extras: Optional[ScoreExtras] = None, pooled: Optional["PooledBlocks"] = None) -> torch.Tensor:
     """Causal attention of each token over the cached keys of its slot up to
     its own position (32-bit arithmetic, any storage type).  ``value_dim``:
     channels of a value head and of a head's output (None: as the keys).
-    ``softcap`` > 0: a score s counts as softcap * tanh(s / softcap)."""
+    ``softcap`` > 0: a score s counts as softcap * tanh(s / softcap).
+    ``pooled``: beside a window, one key and value for every block of tokens
+    that lies wholly before it (``PooledBlocks``), in the same softmax."""
     _dev(q, "q"), _dev(out, "out"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table")
     tokens = q.shape[0]
     value_dim = value_dim or head_dim
@@ -515,6 +566,18 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_
     if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or block_table.dtype != torch.int32:
         raise KernelError("attention: tok_slot, tok_pos and block_table must be int32")
     lib = attention_module(head_dim, value_dim, softcap, extras)
+    if pooled is not None:
+        extras = extras or ScoreExtras()
+        extras.check(heads)
+        pooled.check(k_pages, v_pages, kv_heads, head_dim, value_dim, window)
+        _check(lib, lib.nnis_attention_rows_pooled(q.data_ptr(), _code(q), out.data_ptr(), _code(out), k_pages.data_ptr(),
+                                                   v_pages.data_ptr(), _code(k_pages), block_table.data_ptr(), block_table.shape[1],
+                                                   tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim,
+                                                   int(window), float(scale), int(value_dim), float(softcap), extras.keep_first,
+                                                   _ptr(extras.bias), extras.reach, _ptr(extras.sink), pooled.k_pages.data_ptr(),
+                                                   pooled.v_pages.data_ptr(), pooled.block_table.data_ptr(),
+                                                   pooled.block_table.shape[1], pooled.pool, _stream()))
+        return out
     if extras:
         extras.check(heads)
         _check(lib, lib.nnis_attention_rows_more(q.data_ptr(), _code(q), out.data_ptr(), _code(out), k_pages.data_ptr(),
@@ -1221,7 +1284,8 @@ def prefill_tile_list(new_tokens, first_positions, padded, rows: int):
 
 def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_heads: int, head_dim: int, scale: float,
               window: int = 0, keep_runs: bool = False, tables: Optional[StepTables] = None, plan=None,
-              value_dim: Optional[int] = None, softcap: float = 0.0, extras: Optional[ScoreExtras] = None):
+              value_dim: Optional[int] = None, softcap: float = 0.0, extras: Optional[ScoreExtras] = None,
+              pooled: Optional[PooledBlocks] = None):
     """Attention of the step's tokens over the cache ``view``: bfloat16 with a
     head size in steps of 16 runs on the matrix cores (one kernel for single
     tokens, one for runs of tokens); anything else takes the 32-bit kernel.
@@ -1231,7 +1295,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     (waves, columns) of a step of prompts (``prefill_plan``); None: as those
     functions choose for the step's planned sizes."""
     value_dim = value_dim or head_dim
-    fast = attention_on_matrix_cores(q.dtype, view.k_pages.dtype, head_dim, value_dim, softcap, extras)
+    fast = pooled is None and attention_on_matrix_cores(q.dtype, view.k_pages.dtype, head_dim, value_dim, softcap, extras)
     size = max(head_dim, value_dim)  # what a wave's registers are sized by
     if fast and ctx.decode and heads // kv_heads <= 16 * (4 if size <= 64 else (2 if size <= 128 else 1)):
         splits, waves = plan or decode_plan(ctx.batch, kv_heads, ctx.planned_len, width=heads * value_dim)
@@ -1255,7 +1319,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,
                                       waves, columns, value_dim, softcap, extras)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
-                          kv_heads, head_dim, scale, window, value_dim, softcap, extras)
+                          kv_heads, head_dim, scale, window, value_dim, softcap, extras, pooled)
 
 
 def attention_on_matrix_cores(q_dtype, cache_dtype, head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0,
@@ -1742,3 +1806,212 @@ def head_scale(o: torch.Tensor, gate: torch.Tensor, heads: int) -> torch.Tensor:
     lib = latent()
     _check(lib, lib.nnis_head_scale(o.data_ptr(), _code(o), gate.data_ptr(), tokens, heads, o.shape[1] // heads, _stream()))
     return o
+
+
+# ---------------------------------------------------------------------------
+# sublayers that norm their outputs, gate or pool their heads, or route their tokens
+# ---------------------------------------------------------------------------
+
+def cast_rows(x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[r] = x[rows[r]] (or x[r] without ``rows``) in out's type."""
+    _dev(x, "x"), _dev(out, "out")
+    if x.dim() != 2 or out.dim() != 2 or out.shape[1] != x.shape[1] or (rows is None and out.shape[0] != x.shape[0]):
+        raise KernelError(f"cast_rows: x {tuple(x.shape)} against out {tuple(out.shape)}")
+    if rows is not None:
+        _dev(rows, "rows")
+        if rows.dtype != torch.int32 or rows.numel() < out.shape[0]:
+            raise KernelError("cast_rows: rows must be int32 with one entry per output row")
+    lib = sublayer()
+    _check(lib, lib.nnis_cast_rows(x.data_ptr(), _code(x), out.data_ptr(), _code(out), _ptr(rows), out.shape[0], x.shape[1], _stream()))
+    return out
+
+
+def rms_post_step(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, offset: float, eps: float,
+                  h: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x += y / sqrt(mean(y^2) + eps) * (offset + weight), row by row, in place in the 32-bit stream ``x``; ``h`` (of
+    x's shape, any type) receives the new rows."""
+    _dev(x, "x"), _dev(y, "y"), _dev(weight, "norm weight")
+    if x.dtype != torch.float32 or x.dim() != 2 or y.shape != x.shape or weight.numel() != x.shape[1]:
+        raise KernelError(f"rms_post_step: a float32 stream {tuple(x.shape)} against y {tuple(y.shape)} and a weight of {weight.numel()}")
+    if h is not None:
+        _dev(h, "h")
+        if h.shape != x.shape:
+            raise KernelError(f"rms_post_step: h {tuple(h.shape)} against the stream {tuple(x.shape)}")
+    lib = sublayer()
+    _check(lib, lib.nnis_rms_post_step(x.data_ptr(), y.data_ptr(), _code(y), weight.data_ptr(), _code(weight), float(offset), float(eps),
+                                       _ptr(h), _code(h) if h is not None else 0, x.shape[0], x.shape[1], _stream()))
+    return h
+
+
+def poly_norm(z: torch.Tensor, coefficients: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
+    """out = a N(z) + b N(z^2) + c N(z^3) + e row by row, N(v) = v / sqrt(mean(v^2) + eps); ``coefficients``: float32
+    (a, b, c, e) on the device."""
+    _dev(z, "z"), _dev(coefficients, "coefficients"), _dev(out, "out")
+    if z.dim() != 2 or out.shape != z.shape or coefficients.dtype != torch.float32 or coefficients.numel() != 4:
+        raise KernelError(f"poly_norm: z {tuple(z.shape)}, out {tuple(out.shape)}, four float32 coefficients")
+    lib = sublayer()
+    _check(lib, lib.nnis_poly_norm(z.data_ptr(), _code(z), coefficients.data_ptr(), float(eps), out.data_ptr(), _code(out), z.shape[0],
+                                   z.shape[1], _stream()))
+    return out
+
+
+ROUTE_MOST_OUTPUTS = 1024
+
+
+def route_top(logits: torch.Tensor, correction: Optional[torch.Tensor], experts: int, top: int, gates: torch.Tensor,
+              keep: torch.Tensor):
+    """Scores softmax(logits) [rows, n]; the ``top`` largest of score + correction are chosen.  ``gates`` [rows, experts]
+    gets the score of every chosen output below ``experts`` and 0 elsewhere; ``keep`` [rows] the summed scores of the
+    chosen outputs from ``experts`` on.  All float32."""
+    _dev(logits, "logits"), _dev(gates, "gates"), _dev(keep, "keep")
+    rows, n = logits.shape
+    if logits.dtype != torch.float32 or gates.dtype != torch.float32 or keep.dtype != torch.float32 \
+            or tuple(gates.shape) != (rows, experts) or keep.numel() != rows:
+        raise KernelError(f"route_top: float32 logits {tuple(logits.shape)}, gates {tuple(gates.shape)}, keep {tuple(keep.shape)}")
+    if correction is not None:
+        _dev(correction, "correction")
+        if correction.dtype != torch.float32 or correction.numel() != n:
+            raise KernelError(f"route_top: a float32 correction per output ({n}), got {tuple(correction.shape)} {correction.dtype}")
+    if not (0 < n <= ROUTE_MOST_OUTPUTS and 0 <= experts <= n and 0 < top <= n):
+        raise KernelError(f"route_top: {experts} experts and the {top} largest of {n} outputs (at most {ROUTE_MOST_OUTPUTS})")
+    lib = sublayer()
+    _check(lib, lib.nnis_route_top(logits.data_ptr(), _ptr(correction), rows, n, experts, top, gates.data_ptr(), keep.data_ptr(), _stream()))
+    return gates, keep
+
+
+def routed_act(z: torch.Tensor, gates: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[row, e * ff + c] = gates[row, e] * relu(z[row, e * ff + c])^2 on the experts' fused up projection."""
+    _dev(z, "z"), _dev(gates, "gates"), _dev(out, "out")
+    rows, experts = gates.shape
+    if gates.dtype != torch.float32 or z.dim() != 2 or z.shape[0] != rows or z.shape[1] % max(experts, 1) or out.shape != z.shape:
+        raise KernelError(f"routed_act: z {tuple(z.shape)} and out {tuple(out.shape)} against gates {tuple(gates.shape)}")
+    lib = sublayer()
+    _check(lib, lib.nnis_routed_act(z.data_ptr(), _code(z), gates.data_ptr(), out.data_ptr(), _code(out), rows, experts,
+                                    z.shape[1] // experts, _stream()))
+    return out
+
+
+def rows_axpy(y: torch.Tensor, h: torch.Tensor, keep: torch.Tensor) -> torch.Tensor:
+    """y[row] += keep[row] * h[row]."""
+    _dev(y, "y"), _dev(h, "h"), _dev(keep, "keep")
+    if y.dim() != 2 or h.shape != y.shape or keep.dtype != torch.float32 or keep.numel() != y.shape[0]:
+        raise KernelError(f"rows_axpy: y {tuple(y.shape)}, h {tuple(h.shape)}, a float32 factor per row")
+    lib = sublayer()
+    _check(lib, lib.nnis_rows_axpy(y.data_ptr(), _code(y), h.data_ptr(), _code(h), keep.data_ptr(), y.shape[0], y.shape[1], _stream()))
+    return y
+
+
+def sigmoid_gate(o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """o *= sigmoid(gate) element by element; ``gate``: a view [rows, width] whose rows may be further apart."""
+    _dev(o, "o")
+    if not gate.is_cuda or gate.shape != o.shape or o.dim() != 2 or (gate.shape[1] > 1 and gate.stride(1) != 1):
+        raise KernelError(f"sigmoid_gate: o {tuple(o.shape)} against a gate {tuple(gate.shape)} with adjacent columns")
+    lib = sublayer()
+    _check(lib, lib.nnis_sigmoid_gate(o.data_ptr(), _code(o), gate.data_ptr(), _code(gate), gate.stride(0) if o.shape[0] > 1 else o.shape[1],
+                                      o.shape[0], o.shape[1], _stream()))
+    return o
+
+
+HEAD_NORM_MOST_CHANNELS = 1024
+
+
+def head_norm_write(rows: torch.Tensor, columns, q_out: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                    eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot_dim: int, neighbours: bool,
+                    tok_slot: torch.Tensor, tok_pos: torch.Tensor, k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
+                    block_table: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int, value_dim: int) -> torch.Tensor:
+    """Queries and keys of a fused projection's ``rows`` head by head: an RMS norm over the head with a weight that the
+    heads share (None: no norm), then the rotation of the first ``rot_dim`` channels by the token's position (channel
+    2i with 2i + 1 if ``neighbours``, else i with i + rot_dim / 2); queries to ``q_out``, keys and values into the
+    pages.  ``columns``: (first column of the queries, of the keys, of the values) in a row; with ``k_pages`` None the
+    rows bring queries only."""
+    _dev(rows, "rows"), _dev(q_out, "q_out"), _dev(tok_slot, "tok_slot"), _dev(tok_pos, "tok_pos")
+    tokens = rows.shape[0]
+    q_col, k_col, v_col = columns
+    keys = kv_heads if k_pages is not None else 0
+    need = max(q_col + heads * head_dim, (k_col + keys * head_dim) if keys else 0, (v_col + keys * value_dim) if keys else 0)
+    if rows.dim() != 2 or rows.shape[1] < need or tuple(q_out.shape) != (tokens, heads * head_dim):
+        raise KernelError(f"head_norm_write: rows {tuple(rows.shape)} / q_out {tuple(q_out.shape)} do not fit {heads}+{keys} heads of {head_dim}")
+    if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or tok_slot.numel() < tokens or tok_pos.numel() < tokens:
+        raise KernelError("head_norm_write: tok_slot / tok_pos must be int32 with one entry per token")
+    if head_dim > HEAD_NORM_MOST_CHANNELS:
+        raise KernelError(f"head_norm_write: heads of up to {HEAD_NORM_MOST_CHANNELS} channels, got {head_dim}")
+    w_code = 0
+    for weight in (q_weight, k_weight):
+        if weight is not None:
+            _dev(weight, "head norm weight")
+            if weight.numel() != head_dim:
+                raise KernelError(f"head_norm_write: a norm weight of {weight.numel()} for heads of {head_dim}")
+            w_code = _code(weight)
+    if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
+        raise KernelError("head_norm_write: the two norm weights differ in type")
+    table_positions = 0
+    if cos is not None:
+        _dev(cos, "cos"), _dev(sin, "sin")
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] != rot_dim // 2:
+            raise KernelError(f"head_norm_write: tables {tuple(cos.shape)} do not fit rot_dim {rot_dim} in float32")
+        table_positions = cos.shape[0]
+    max_pages = cache_code = 0
+    if keys:
+        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table")
+        if not _pages_fit(k_pages, v_pages, kv_heads, head_dim, value_dim):
+            raise KernelError(f"head_norm_write: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2:
+            raise KernelError("head_norm_write: block_table must be int32 [slots, pages]")
+        max_pages, cache_code = block_table.shape[1], _code(k_pages)
+    lib = sublayer()
+    _check(lib, lib.nnis_head_norm_write(rows.data_ptr(), _code(rows), rows.stride(0) if tokens > 1 else rows.shape[1], q_col,
+                                         k_col if keys else -1, v_col if keys else -1, q_out.data_ptr(), _code(q_out), _ptr(q_weight),
+                                         _ptr(k_weight), w_code, float(eps), _ptr(cos), _ptr(sin), table_positions, int(rot_dim),
+                                         1 if neighbours else 0, tok_slot.data_ptr(), tok_pos.data_ptr(), _ptr(k_pages) if keys else None,
+                                         _ptr(v_pages) if keys else None, cache_code, _ptr(block_table) if keys else None, max_pages,
+                                         tokens, heads, keys, head_dim, int(value_dim), _stream()))
+    return q_out
+
+
+def pool_blocks(k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor, pooled: PooledBlocks, tok_slot: torch.Tensor,
+                tok_pos: torch.Tensor, tokens: int, kv_heads: int, head_dim: int, value_dim: int) -> None:
+    """For every token of the step that completes a block of ``pooled.pool`` tokens of its sequence: the mean of the
+    block's keys and the mean of its values, as the pages hold them, into the block's entry of ``pooled``."""
+    for t, what in ((k_pages, "k_pages"), (v_pages, "v_pages"), (block_table, "block_table"), (tok_slot, "tok_slot"), (tok_pos, "tok_pos")):
+        _dev(t, what)
+    pooled.check(k_pages, v_pages, kv_heads, head_dim, value_dim, window=1)
+    if not _pages_fit(k_pages, v_pages, kv_heads, head_dim, value_dim):
+        raise KernelError(f"pool_blocks: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
+    if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or tok_slot.numel() < tokens or tok_pos.numel() < tokens:
+        raise KernelError("pool_blocks: tok_slot / tok_pos must be int32 with one entry per token")
+    lib = sublayer()
+    _check(lib, lib.nnis_pool_blocks(k_pages.data_ptr(), v_pages.data_ptr(), _code(k_pages), block_table.data_ptr(), block_table.shape[1],
+                                     pooled.k_pages.data_ptr(), pooled.v_pages.data_ptr(), pooled.block_table.data_ptr(),
+                                     pooled.block_table.shape[1], tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, kv_heads, head_dim,
+                                     int(value_dim), pooled.pool, _stream()))
+
+
+def min_gru(rows: torch.Tensor, z_bias: Optional[torch.Tensor], x_bias: Optional[torch.Tensor], state: torch.Tensor, ctx,
+            out: torch.Tensor) -> torch.Tensor:
+    """The minGRU recurrence over each sequence's tokens, from and into ``state`` (float32 [slots, width]): with ``rows``
+    [tokens, 3 * width] = (zp | up | g): z = sigmoid(zp + z_bias), u = up + x_bias, c = u + 1/2 where u >= 0 and
+    sigmoid(u) below, S <- (1 - z) S + z c, out = S * silu(g)."""
+    _dev(rows, "rows"), _dev(state, "state"), _dev(out, "out")
+    tokens, width = out.shape
+    if rows.dim() != 2 or rows.shape[0] != tokens or rows.shape[1] < 3 * width:
+        raise KernelError(f"min_gru: rows {tuple(rows.shape)} do not hold three times the {width} channels of out {tuple(out.shape)}")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (width,):
+        raise KernelError(f"min_gru: state must be float32 [slots, {width}], got {tuple(state.shape)} {state.dtype}")
+    if (z_bias is None) != (x_bias is None):
+        raise KernelError("min_gru: both biases or none")
+    if z_bias is not None:
+        _dev(z_bias, "z_bias"), _dev(x_bias, "x_bias")
+        if z_bias.numel() != width or x_bias.numel() != width or z_bias.dtype != x_bias.dtype:
+            raise KernelError("min_gru: the biases have one entry per channel and one type")
+    _step_arrays(ctx, "min_gru")
+    piece, pieces = run_pieces(ctx, width * 8)
+    decay = ends = None
+    if pieces > 1:
+        scratch = torch.empty(2, ctx.batch * pieces * width, dtype=torch.float32, device=rows.device)
+        decay, ends = scratch[0], scratch[1]
+    lib = recurrent()
+    _check(lib, lib.nnis_min_gru(rows.data_ptr(), _code(rows), rows.stride(0) if tokens > 1 else rows.shape[1], _ptr(z_bias), _ptr(x_bias),
+                                 _code(z_bias) if z_bias is not None else 0, state.data_ptr(), ctx.seq_slot.data_ptr(),
+                                 ctx.seq_start.data_ptr(), ctx.batch, width, out.data_ptr(), _code(out), piece, pieces, _ptr(decay),
+                                 _ptr(ends), _stream()))
+    return out

@@ -110,6 +110,12 @@ class DecoderModel:
                 requests.append((index, self.layers[entry.layer].cache_request()))
             else:
                 shared[index] = entry.reads_cache_of
+                # what the layer keeps of its own beside the cache it reads (pooled blocks of another size, say): its
+                # view is then the pair (the other entry's view, its own)
+                beside = getattr(self.layers[entry.layer], "cache_request_beside", None)
+                beside = beside() if beside is not None else None
+                if beside is not None:
+                    requests.append((index, beside))
         return requests, shared
 
     # ---- forward -------------------------------------------------------------

@@ -228,3 +228,165 @@ class CausalSelfAttention(Mixer):
 
 
 register_part("mixer", "causal_attention", CausalSelfAttention)
+
+
+class GatedWindowAttention(Mixer):
+    """Grouped attention whose queries and keys are normed head by head, whose
+    window may come with pooled blocks, and whose heads are gated:
+
+        q = rot(R(Wq h, wq)),  k = rot(R(Wk h, wk)),  v = Wv h       R: RMS norm over a head's channels, one weight for
+                                                                     all heads; rot: channel 2i turns with 2i + 1
+        s(i, j) = cap * tanh(q_i . k_j * scale / cap)                0 <= i - j < window
+        s(i, b) the same with the mean key of block b                b * pool + pool - 1 <= i - window
+        p = exp(s) / (sum_j exp s(i, j) + sum_b exp s(i, b) + exp(sink_head))
+        out = Wo (concat_heads(sum p v) * sigmoid(Wg h))
+
+    A block's key and value are the means of its ``pool`` tokens' keys and
+    values as the cache holds them; they live in pages of their own, one entry
+    a block (``KVRequest.every``), written by the step that completes the
+    block.  Tokens that have left the window and whose block is not complete
+    before it are not seen.  Each of cap, window, pool and rotation is off when
+    zero or None.  ``own_kv`` False: the layer has no keys and values; it reads
+    those of the schedule entry that the model names (``reads_cache_of``) with
+    its own queries and mask, and that entry's pooled blocks if their size
+    (``source_pool``) is this layer's, else it keeps pooled blocks of its own
+    beside them (``cache_request_beside``)."""
+
+    graph_safe = True
+
+    def __init__(self, width, heads, kv_heads, head_dim, value_dim, scale, eps, q, o, gate, q_norm, sink, k=None, v=None, k_norm=None,
+                 position=None, positions=None, window=None, pool=None, softcap=None, own_kv=True, source_pool=None):
+        if heads % kv_heads != 0:
+            raise InvalidInput(f"{heads} query heads do not divide into {kv_heads} key/value heads")
+        self.width, self.heads, self.kv_heads = int(width), int(heads), int(kv_heads)
+        self.head_dim, self.value_dim = int(head_dim), int(value_dim)
+        self.scale, self.eps = float(scale), float(eps)
+        if min(self.width, self.heads, self.head_dim, self.value_dim) <= 0 or not self.scale > 0.0:
+            raise InvalidInput("attention needs positive sizes and a positive scale")
+        self.softcap = 0.0 if not softcap else float(softcap)
+        self.window = 0 if not window else int(window)
+        self.pool = 0 if not pool else int(pool)
+        if self.pool and not self.window:
+            raise InvalidInput(f"pooled blocks of {self.pool} tokens stand beside a window only")
+        self.own_kv = bool(own_kv)
+        self.source_pool = 0 if not source_pool else int(source_pool)
+        if self.own_kv and (k is None or v is None or k_norm is None):
+            raise InvalidInput("a layer with keys and values of its own names their projections and the keys' norm")
+        self.names = {"q": q, "k": k, "v": v, "o": o, "gate": gate, "q_norm": q_norm, "k_norm": k_norm, "sink": sink}
+        self.position = None
+        if position is not None:
+            if positions is None or position not in positions:
+                raise InvalidInput(f"attention names position encoding {position!r}, which the model does not define")
+            self.position = positions[position]
+            if getattr(self.position, "pairing", None) != "neighbours":
+                raise InvalidInput("this attention turns neighbouring channels: the position encoding must say so")
+        self.proj = self.out = self.q_norm = self.k_norm = self.extras = None
+
+    def tensors(self):
+        n, qw, ow = self.names, self.heads * self.head_dim, self.heads * self.value_dim
+        out = [TensorSpec(n["q"], (qw, self.width)), TensorSpec(n["q_norm"], (self.head_dim,), init="gain"),
+               TensorSpec(n["sink"], (self.heads,), init="small"), TensorSpec(n["gate"], (ow, self.width)),
+               TensorSpec(n["o"], (self.width, ow))]
+        if self.own_kv:
+            out += [TensorSpec(n["k"], (self.kv_heads * self.head_dim, self.width)),
+                    TensorSpec(n["v"], (self.kv_heads * self.value_dim, self.width)),
+                    TensorSpec(n["k_norm"], (self.head_dim,), init="gain")]
+        return out
+
+    def bind(self, weights, rt):
+        n = self.names
+        # one projection for everything that reads the mixer's input: rows [q | k | v | gate] (or [q | gate])
+        parts = [weights[n["q"]]] + ([weights[n["k"]], weights[n["v"]]] if self.own_kv else []) + [weights[n["gate"]]]
+        self.proj = Projection(torch.cat(parts, dim=0), rt)
+        self.out = Projection(weights[n["o"]], rt)
+        self.q_norm = weights[n["q_norm"]].float().contiguous()
+        self.k_norm = weights[n["k_norm"]].float().contiguous() if self.own_kv else None
+        self.extras = rt.ops.ScoreExtras(0, None, weights[n["sink"]].float().contiguous())
+        qw = self.heads * self.head_dim
+        kw, vw = (self.kv_heads * self.head_dim, self.kv_heads * self.value_dim) if self.own_kv else (0, 0)
+        self.columns = (0, qw, qw + kw)
+        self.gate_column = qw + kw + vw
+
+    def weight_bytes(self):
+        return self.proj.weight_bytes() + self.out.weight_bytes()
+
+    def _pooled_request(self):
+        return KVRequest(self.kv_heads, self.head_dim, None, None if self.value_dim == self.head_dim else self.value_dim, every=self.pool)
+
+    def cache_request(self):
+        main = KVRequest(self.kv_heads, self.head_dim, None, None if self.value_dim == self.head_dim else self.value_dim)
+        return (main, self._pooled_request() if self.pool else None)
+
+    def cache_request_beside(self):
+        """What this layer keeps while its keys and values are another entry's: pooled blocks, if it sees any and the
+        other entry keeps none of this size."""
+        if self.own_kv or not self.pool or self.pool == self.source_pool:
+            return None
+        return self._pooled_request()
+
+    def check(self, rt):
+        # (pooled blocks take the row kernel, which carries heads beyond the matrix-core kernels' sizes too)
+        rt.ops.attention_check(self.head_dim, self.value_dim)
+        rot_dim = getattr(self.position, "rot_dim", 0)
+        if rot_dim > self.head_dim:
+            raise InvalidInput(f"a rotation of {rot_dim} channels does not fit heads of {self.head_dim}")
+
+    def _matrix_cores(self, rt) -> bool:
+        return not self.pool and rt.ops.attention_on_matrix_cores(rt.dtype, rt.dtype, self.head_dim, self.value_dim, self.softcap, self.extras)
+
+    def decode_plan(self, batch, longest, rt):
+        if not self._matrix_cores(rt):
+            return None
+        return rt.ops.decode_plan(batch, self.kv_heads, longest, width=self.heads * self.value_dim)
+
+    def prompt_plan(self, batch, rows, longest, rt):
+        if not self._matrix_cores(rt):
+            return None
+        return rt.ops.prefill_plan(longest, rows, self.heads, max(self.head_dim, self.value_dim), self.kv_heads)
+
+    def held_buffers(self, rt):
+        held = rt.ops.decode_scratch_held(rt.device)
+        return [] if held is None else [held]
+
+    def _views(self, view):
+        """(keys and values, pooled blocks or None, whether this layer writes the pooled blocks)."""
+        if isinstance(view[0], tuple):  # another entry's views, and pooled blocks of this layer's own beside them
+            return view[0][0], view[1], True
+        main, pooled = view
+        if not self.pool:
+            return main, None, False
+        if pooled is None:
+            raise InvalidInput("this layer sees pooled blocks, but its cache keeps none of its size")
+        return main, pooled, not pooled.read_only
+
+    def forward(self, x, ctx, view, rt):
+        main, pooled_view, writes_pooled = self._views(view)
+        if self.own_kv == main.read_only:
+            raise InvalidInput("a layer with keys and values of its own writes them; one without reads another's")
+        tokens = x.shape[0]
+        rows = self.proj(x, rt)
+        tables = self.position.rotary() if self.position is not None else None
+        q = rt.ops.head_norm_write(
+            rows, self.columns, rt.empty(tokens, self.heads * self.head_dim), self.q_norm, self.k_norm, self.eps,
+            tables.cos if tables else None, tables.sin if tables else None, tables.rot_dim if tables else 0, True,
+            ctx.tok_slot, ctx.tok_pos, main.k_pages if self.own_kv else None, main.v_pages if self.own_kv else None,
+            main.block_table if self.own_kv else None, self.heads, self.kv_heads, self.head_dim, self.value_dim)
+        pooled = None
+        if pooled_view is not None:
+            pooled = rt.ops.PooledBlocks(pooled_view.k_pages, pooled_view.v_pages, pooled_view.block_table, self.pool)
+            if writes_pooled:
+                rt.ops.pool_blocks(main.k_pages, main.v_pages, main.block_table, pooled, ctx.tok_slot, ctx.tok_pos, tokens,
+                                   self.kv_heads, self.head_dim, self.value_dim)
+        plan = None
+        if self._matrix_cores(rt) and main.k_pages.dtype == torch.bfloat16:
+            plan = (self.decode_plan(ctx.batch, ctx.planned_len, rt) if ctx.decode
+                    else self.prompt_plan(ctx.batch, ctx.planned_rows, ctx.planned_len, rt))
+        attn = rt.ops.attention(q, rt.empty(tokens, self.heads * self.value_dim), main, ctx, self.heads, self.kv_heads, self.head_dim,
+                                self.scale, self.window, plan=plan, value_dim=self.value_dim, softcap=self.softcap,
+                                extras=self.extras, pooled=pooled)
+        gate = rows[:, self.gate_column:self.gate_column + self.heads * self.value_dim]
+        rt.ops.sigmoid_gate(attn, gate)
+        return self.out(attn, rt)
+
+
+register_part("mixer", "gated_window_attention", GatedWindowAttention)

@@ -76,12 +76,17 @@ class TensorSpec:
 class KVRequest:
     """Keys and values of every token (``window is None``) or of the last
     ``window`` tokens, for ``kv_heads`` heads whose keys have ``head_dim``
-    channels and whose values ``value_dim`` (None: as many as the keys)."""
+    channels and whose values ``value_dim`` (None: as many as the keys).
+    ``every`` > 1: one entry for every ``every`` tokens of a sequence, the
+    last tokens that do not fill one left out (what a mixer keeps of whole
+    blocks of tokens): a sequence of n tokens holds n // every entries, in
+    pages and a block table of the group's own."""
 
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
+    every: int = 1
 
     @property
     def value_head_dim(self) -> int:

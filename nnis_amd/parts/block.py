@@ -298,6 +298,86 @@ class PrePostNormBlock(Block):
         return x, PostNormed(y, post)
 
 
+class PostNormBlock(Block):
+    """A layer whose sublayers read the stream as it is and are normed on their way out only:
+
+        x <- x + norm1(mixer(x));   x <- x + norm2(feed_forward(x))
+
+    (the second line only with a feed-forward).  The norm on the way out, the sum into the 32-bit stream and the
+    stream's rows in the activation type, which the next sublayer reads, are one kernel (``Norm.post_step``); the rows
+    behind the layer's last sublayer are handed to a block of this kind that comes next (``PreparedRows``)."""
+
+    def __init__(self, width, norm1, mixer, norm2=None, feed_forward=None, positions=None):
+        self.width = int(width)
+        if (feed_forward is None) != (norm2 is None):
+            raise InvalidInput("a feed-forward comes with its norm, or neither")
+        self.entry = build_part("norm", {"kind": "none", "width": self.width})  # how this block reads the stream
+        self.norm1 = build_part("norm", norm1)
+        self.mixer = build_part("mixer", mixer, positions=positions)
+        self.norm2 = build_part("norm", norm2) if norm2 is not None else None
+        self.feed_forward = build_part("feed_forward", feed_forward) if feed_forward is not None else None
+        for norm in (self.norm1, self.norm2):
+            if norm is not None and not hasattr(norm, "post_step"):
+                raise InvalidInput("a block that norms its sublayers' outputs needs norms that bring them into the stream (post_step)")
+        self._parts = [part for part in (self.norm1, self.mixer, self.norm2, self.feed_forward) if part is not None]
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self._parts)
+
+    def tensors(self):
+        return [spec for part in self._parts for spec in part.tensors()]
+
+    def bind(self, weights, rt):
+        for part in self._parts:
+            part.bind(weights, rt)
+
+    def weight_bytes(self):
+        return sum(part.weight_bytes() for part in self._parts)
+
+    def cache_request(self):
+        return self.mixer.cache_request()
+
+    def cache_request_beside(self):
+        """What the mixer keeps of its own while its keys and values are another entry's (see ``Mixer.cache_request_beside``)."""
+        return self.mixer.cache_request_beside() if hasattr(self.mixer, "cache_request_beside") else None
+
+    def check(self, rt):
+        for part in self._parts:
+            part.check(rt)
+
+    def decode_plan(self, batch, longest, rt):
+        return _joined(part.decode_plan(batch, longest, rt) for part in self._parts)
+
+    def prompt_plan(self, batch, rows, longest, rt):
+        return _joined(part.prompt_plan(batch, rows, longest, rt) for part in self._parts)
+
+    def held_buffers(self, rt):
+        return [buffer for part in self._parts for buffer in part.held_buffers(rt)]
+
+    @property
+    def entry_norm(self):
+        return self.entry
+
+    def forward(self, stream, ctx, view, rt, following=None):
+        """stream: (x, pending), or the stream with its rows made already (``PreparedRows`` of a norm of kind
+        ``none``).  following: the next block's first norm; if that reads the stream as it is, the rows go with it."""
+        if isinstance(stream, PreparedRows):
+            if type(stream.norm) is not type(self.entry):
+                raise ValueError("the rows handed to a block are not the stream's own")
+            x, h = stream.x, stream.h
+        else:
+            x, pending = stream
+            if isinstance(pending, PostNormed):
+                pending = pending.materialize(rt)
+            if pending is not None:
+                raise InvalidInput("a block that reads the stream as it is takes it with nothing left to add")
+            h = self.entry.forward(x, rt)
+        h = self.norm1.post_step(x, self.mixer.forward(h, ctx, view, rt), rt)
+        if self.feed_forward is not None:
+            h = self.norm2.post_step(x, self.feed_forward.forward(h, ctx, rt), rt)
+        if following is not None and type(following) is type(self.entry):
+            return PreparedRows(following, x, h)
+        return x, None
+
+
 def _noise(spec, generator):
     return torch.randn(tuple(spec.shape), generator=generator, dtype=torch.float32)
 
@@ -309,3 +389,4 @@ register_init_rule("stream_share", lambda spec, generator, dtype: (0.5 + 0.25 * 
 register_part("block", "pre_norm", PreNormBlock)
 register_part("block", "hyper_connections", HyperConnectionBlock)
 register_part("block", "pre_post_norm", PrePostNormBlock)
+register_part("block", "post_norm", PostNormBlock)

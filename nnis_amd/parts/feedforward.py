@@ -8,7 +8,8 @@ from __future__ import annotations
 
 import torch
 
-from ..errors import Unsupported
+from ..errors import InvalidInput, Unsupported
+from ..weights.random_init import register_init_rule
 from .base import FeedForward, TensorSpec, register_part
 from .linear import Projection
 
@@ -67,3 +68,95 @@ class GatedFeedForward(FeedForward):
 
 
 register_part("feed_forward", "gated", GatedFeedForward)
+
+
+class PolyNormFeedForward(FeedForward):
+    """down(act(up x)) with act(z) = a N(z) + b N(z^2) + c N(z^3) + e: powers element by element, N a division of a
+    token's inner row by its root mean square (eps inside the root); (a, b, c, e) are the four numbers of ``act``.
+    The statistics and the polynomial are 32-bit."""
+
+    graph_safe = True
+
+    def __init__(self, width, inner, eps, up, down, act):
+        self.width, self.inner, self.eps = int(width), int(inner), float(eps)
+        self.names = {"up": up, "down": down, "act": act}
+        self.up = self.down = self.coefficients = None
+
+    def tensors(self):
+        return [TensorSpec(self.names["up"], (self.inner, self.width)), TensorSpec(self.names["down"], (self.width, self.inner)),
+                TensorSpec(self.names["act"], (4,), init="poly_coefficients")]
+
+    def bind(self, weights, rt):
+        self.up = Projection(weights[self.names["up"]], rt)
+        self.down = Projection(weights[self.names["down"]], rt)
+        self.coefficients = weights[self.names["act"]].float().contiguous()
+
+    def weight_bytes(self):
+        return self.up.weight_bytes() + self.down.weight_bytes() + 16
+
+    def forward(self, x, ctx, rt):
+        z = self.up(x, rt)
+        return self.down(rt.ops.poly_norm(z, self.coefficients, self.eps, rt.empty(x.shape[0], self.inner)), rt)
+
+
+class RoutedFeedForward(FeedForward):
+    """A mixture of ``experts`` small feed-forwards, down_e(relu(up_e x)^2), of which a token uses ``top``:
+
+        s = softmax(W_r x) over experts + identity outputs       32-bit
+        chosen = the ``top`` largest of s + correction           (the lower index on a tie)
+        out = sum over chosen e of s_e * expert_e(x),            expert_e(x) = x for the last ``identity`` outputs
+
+    The weights are the scores themselves, not renormalised; ``correction`` (a tensor's name or None) enters the
+    choice only.  The experts' up projections are one product over all experts, gated row by row with the scores
+    (zero for the experts not chosen) before one down projection over all of them."""
+
+    graph_safe = True
+
+    def __init__(self, width, inner, experts, top, router, up, down, identity=0, correction=None):
+        """``up`` and ``down``: names with ``{}`` in the expert's place."""
+        self.width, self.inner, self.experts, self.top, self.identity = int(width), int(inner), int(experts), int(top), int(identity or 0)
+        if min(self.width, self.inner, self.experts, self.top) <= 0 or self.identity < 0 or self.top > self.experts + self.identity:
+            raise InvalidInput(f"a router of {experts} experts and {identity} identity outputs cannot choose {top}")
+        self.names = {"router": router, "up": up, "down": down, "correction": correction}
+
+    def tensors(self):
+        n, outputs = self.names, self.experts + self.identity
+        out = [TensorSpec(n["router"], (outputs, self.width), init="router")]
+        if n["correction"]:
+            out.append(TensorSpec(n["correction"], (outputs,), init="small"))
+        for e in range(self.experts):
+            out += [TensorSpec(n["up"].format(e), (self.inner, self.width)), TensorSpec(n["down"].format(e), (self.width, self.inner))]
+        return out
+
+    def check(self, rt):
+        if self.experts + self.identity > rt.ops.ROUTE_MOST_OUTPUTS:
+            raise Unsupported(f"the router kernel takes up to {rt.ops.ROUTE_MOST_OUTPUTS} outputs, got {self.experts + self.identity}")
+
+    def bind(self, weights, rt):
+        n = self.names
+        self.router = weights[n["router"]].float().contiguous()  # its logits are a 32-bit product under either runtime
+        self.correction = weights[n["correction"]].float().contiguous() if n["correction"] else None
+        self.up = Projection(torch.cat([weights[n["up"].format(e)] for e in range(self.experts)], dim=0), rt)
+        self.down = Projection(torch.cat([weights[n["down"].format(e)] for e in range(self.experts)], dim=1), rt)
+
+    def weight_bytes(self):
+        return self.up.weight_bytes() + self.down.weight_bytes() + self.router.numel() * 4
+
+    def forward(self, x, ctx, rt):
+        tokens = x.shape[0]
+        logits = rt.ops.gemm_ordered(x, self.router, rt.empty(tokens, self.experts + self.identity, dtype=torch.float32))
+        gates, keep = rt.ops.route_top(logits, self.correction, self.experts, self.top,
+                                       rt.empty(tokens, self.experts, dtype=torch.float32), rt.empty(tokens, dtype=torch.float32))
+        z = self.up(x, rt)
+        y = self.down(rt.ops.routed_act(z, gates, rt.empty(tokens, self.experts * self.inner)), rt)
+        if self.identity:
+            rt.ops.rows_axpy(y, x, keep)
+        return y
+
+
+# what a random model draws: coefficients of a size that matters, router rows that spread the scores
+register_init_rule("poly_coefficients", lambda spec, generator, dtype: (0.5 + 0.25 * torch.randn(tuple(spec.shape), generator=generator)).to(dtype),
+                   replace=True)
+register_init_rule("router", lambda spec, generator, dtype: (0.3 * torch.randn(tuple(spec.shape), generator=generator)).to(dtype), replace=True)
+register_part("feed_forward", "poly_norm", PolyNormFeedForward)
+register_part("feed_forward", "routed", RoutedFeedForward)

@@ -1,5 +1,6 @@
 """RMSNorm with a per-channel weight: y = x / sqrt(mean(x^2) + eps) * w
-(/root/reference/crates/nnis-model/src/kernels.rs:15-48)."""
+(/root/reference/crates/nnis-model/src/kernels.rs:15-48); with ``offset`` the
+stored weight lies around zero and the gain is offset + w."""
 
 from __future__ import annotations
 
@@ -13,17 +14,24 @@ class RMSNorm(Norm):
     graph_safe = True
     fusable_rms = True  # ``weight`` and ``eps`` are all a projection kernel needs to apply this norm itself
 
-    def __init__(self, width: int, eps: float, weight: str):
+    def __init__(self, width: int, eps: float, weight: str, offset: float = 0.0):
+        """``offset``: the gain is offset + weight (a weight stored around zero has an offset of 1); the sum is made
+        once, in 32-bit, when the weights are bound, and such a norm is not taken into a projection's kernel."""
         self.width = int(width)
         self.eps = float(eps)
         self.weight_name = weight
+        self.offset = float(offset)
         self.weight = None
+        if self.offset:
+            self.fusable_rms = False
 
     def tensors(self):
-        return [TensorSpec(self.weight_name, (self.width,), init="gain")]
+        return [TensorSpec(self.weight_name, (self.width,), init="small" if self.offset else "gain")]
 
     def bind(self, weights, rt):
         self.weight = weights[self.weight_name].contiguous()
+        if self.offset:
+            self.weight = (self.weight.float() + self.offset).contiguous()
 
     def weight_bytes(self):
         return self.weight.numel() * self.weight.element_size()
@@ -38,8 +46,41 @@ class RMSNorm(Norm):
     def add_forward(self, residual, delta, rt, rows=None):
         return rt.ops.rmsnorm(residual, self.weight, self.eps, self._out(residual, rt, rows), delta=delta, rows=rows)
 
+    def post_step(self, x, y, rt):
+        """x += this norm of y, in place in the 32-bit stream; returns the new rows in the activation type (the stream
+        itself under a 32-bit runtime): what a sublayer that reads the stream un-normed takes next."""
+        if rt.dtype == torch.float32:
+            rt.ops.rms_post_step(x, y, self.weight, 0.0, self.eps)
+            return x
+        return rt.ops.rms_post_step(x, y, self.weight, 0.0, self.eps, h=rt.empty(x.shape[0], self.width))
 
+
+register_init_rule("small", lambda spec, generator, dtype: (0.1 * torch.randn(tuple(spec.shape), generator=generator)).to(dtype),
+                   replace=True)
 register_part("norm", "rms", RMSNorm)
+
+
+class NoNorm(Norm):
+    """The stream's rows as they are, in the activation type: what a sublayer
+    reads that is normed on its way out only.  Under a 32-bit runtime that is
+    the stream itself."""
+
+    graph_safe = True
+
+    def __init__(self, width: int):
+        self.width = int(width)
+
+    def forward(self, x, rt, rows=None):
+        if rows is None and x.dtype == rt.dtype:
+            return x
+        count = x.shape[0] if rows is None else rows.shape[0]
+        return rt.ops.cast_rows(x, rt.empty(count, self.width), rows)
+
+    def add_forward(self, residual, delta, rt, rows=None):
+        raise NotImplementedError("a stream that is read as it is has nothing left to add")
+
+
+register_part("norm", "none", NoNorm)
 
 
 class LayerNorm(Norm):

@@ -166,6 +166,51 @@ class GatedLinearAttention(Mixer):
         return self.out(gated, rt)
 
 
+class MinGRU(Mixer):
+    """A gated recurrence whose gates read the current token only.  With C channels:
+
+        z = sigmoid(W_z h + b_z),   u = W_x h + b_x,   c = u + 1/2 where u >= 0, sigmoid(u) below
+        S <- (1 - z) S + z c                              element by element
+        out = W_o (S * silu(W_g h))
+
+    State per sequence: S [C], 32-bit, zero at the start.  The three projections of the input are one product; the
+    gates, the candidate and the recurrence are 32-bit under either runtime."""
+
+    graph_safe = True
+
+    def __init__(self, width, channels, z, z_bias, x, x_bias, g, o):
+        self.width, self.channels = int(width), int(channels)
+        if min(self.width, self.channels) <= 0:
+            raise InvalidInput("a minGRU needs positive sizes")
+        self.names = dict(z=z, z_bias=z_bias, x=x, x_bias=x_bias, g=g, o=o)
+
+    def tensors(self):
+        C, n = self.channels, self.names
+        return [TensorSpec(n["z"], (C, self.width)), TensorSpec(n["z_bias"], (C,), init="small"),
+                TensorSpec(n["x"], (C, self.width)), TensorSpec(n["x_bias"], (C,), init="small"),
+                TensorSpec(n["g"], (C, self.width)), TensorSpec(n["o"], (self.width, C))]
+
+    def bind(self, weights, rt):
+        n = self.names
+        self.zxg = Projection(torch.cat([weights[n[key]] for key in ("z", "x", "g")], dim=0), rt)
+        self.z_bias = weights[n["z_bias"]].float().contiguous()
+        self.x_bias = weights[n["x_bias"]].float().contiguous()
+        self.out = Projection(weights[n["o"]], rt)
+
+    def weight_bytes(self):
+        return self.zxg.weight_bytes() + self.out.weight_bytes() + 8 * self.channels
+
+    def cache_request(self):
+        return StateRequest((self.channels,))
+
+    def forward(self, x, ctx, view, rt):
+        if view.read_only:
+            raise Unsupported("a minGRU cannot read another layer's state")
+        rows = self.zxg(x, rt)
+        y = rt.ops.min_gru(rows, self.z_bias, self.x_bias, view.state, ctx, rt.empty(x.shape[0], self.channels))
+        return self.out(y, rt)
+
+
 class SideBySide(Mixer):
     """Several mixers that read the same input; each output is divided by its
     root mean square over the model width and multiplied by a weight of its
@@ -268,4 +313,5 @@ register_init_rule("decay_bias", lambda spec, generator, dtype: (2.0 + _noise(sp
 
 register_part("mixer", "selective_scan", SelectiveScan)
 register_part("mixer", "gated_linear_attention", GatedLinearAttention)
+register_part("mixer", "min_gru", MinGRU)
 register_part("mixer", "side_by_side", SideBySide)

@@ -8,20 +8,38 @@ rounded once, which is what a correctly rounded 32-bit routine returns.
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 from ..errors import InvalidInput
 from .base import PositionEncoding, RotaryTables, register_part
 
 
-def rotary_tables(positions: int, rot_dim: int, theta: float, angles: str = "float32"):
+def bend_frequencies(inv_freq: torch.Tensor, factor: float, low: float, high: float, original: float) -> torch.Tensor:
+    """Frequencies bent by their wavelength l = 2 pi / f: f stays where l <
+    original / high, becomes f / factor where l > original / low, and between
+    the two (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+    f = inv_freq.to(torch.float64)
+    length = 2.0 * math.pi / f
+    s = (original / length - low) / (high - low)
+    blended = (1.0 - s) * f / factor + s * f
+    return torch.where(length < original / high, f, torch.where(length > original / low, f / factor, blended))
+
+
+def rotary_tables(positions: int, rot_dim: int, theta: float, angles: str = "float32", scaling=None):
     """``angles``: "float32" rounds the frequencies and the angles to 32-bit as
     the reference does; "float64" takes frequency i as theta^(-2i / rot_dim) and
-    the angle as position x frequency in 64-bit, and rounds cosine and sine only."""
+    the angle as position x frequency in 64-bit, and rounds cosine and sine only.
+    ``scaling``: (factor, low, high, original) of ``bend_frequencies``, with 64-bit angles only."""
     half = rot_dim // 2
+    if scaling is not None and angles != "float64":
+        raise InvalidInput("bent frequencies are made with 64-bit angles")
     if angles == "float64":
         pair = torch.arange(half, dtype=torch.float64)
         inv_freq = torch.pow(torch.tensor(float(theta), dtype=torch.float64), -2.0 * pair / float(rot_dim))
+        if scaling is not None:
+            inv_freq = bend_frequencies(inv_freq, *[float(value) for value in scaling])
         angle = torch.arange(positions, dtype=torch.float64)[:, None] * inv_freq[None, :]
         return torch.cos(angle).to(torch.float32), torch.sin(angle).to(torch.float32)
     pair = torch.arange(half, dtype=torch.float32)
@@ -39,9 +57,11 @@ class RotaryHalf(PositionEncoding):
     graph_safe = True
     pairing = "halves"  # channel i turns with channel i + rot_dim / 2
 
-    def __init__(self, rot_dim: int, theta: float, max_positions: int = None, angles: str = "float32"):
+    def __init__(self, rot_dim: int, theta: float, max_positions: int = None, angles: str = "float32", scaling=None):
         """``max_positions`` None: the model names no last position; the tables
-        are made as long as the engine's cache lets a sequence grow (``reach``)."""
+        are made as long as the engine's cache lets a sequence grow (``reach``).
+        ``scaling``: (factor, low, high, original), frequencies bent by their
+        wavelength (``bend_frequencies``)."""
         if rot_dim <= 0 or rot_dim % 2 != 0:
             raise InvalidInput(f"rotary dimension must be even and positive; got {rot_dim}")
         if angles not in ("float32", "float64"):
@@ -50,6 +70,9 @@ class RotaryHalf(PositionEncoding):
         self.theta = float(theta)
         self.max_positions = None if max_positions is None else int(max_positions)
         self.angles = angles
+        self.scaling = None if scaling is None else tuple(float(value) for value in scaling)
+        if self.scaling is not None and len(self.scaling) != 4:
+            raise InvalidInput(f"bent frequencies take (factor, low, high, original); got {scaling!r}")
         self._tables = None
         self._device = None
         self._kept = []
@@ -59,7 +82,7 @@ class RotaryHalf(PositionEncoding):
         self._make(self.max_positions or 64)
 
     def _make(self, positions: int) -> None:
-        cos, sin = rotary_tables(positions, self.rot_dim, self.theta, self.angles)
+        cos, sin = rotary_tables(positions, self.rot_dim, self.theta, self.angles, self.scaling)
         self._tables = RotaryTables(cos.to(self._device).contiguous(), sin.to(self._device).contiguous(), self.rot_dim)
 
     def reach(self, positions: int) -> None:

@@ -56,6 +56,14 @@ constexpr int HDR = NNIS_REG_DIM;
 #ifndef NNIS_SCORE_EXTRAS
 #define NNIS_SCORE_EXTRAS 0
 #endif
+// 1 (with the extras): the matrix-core kernels also take pooled blocks beside a window (see AttnArgs); compiled in,
+// so that the kernels of modules without them stay the code they are
+#ifndef NNIS_POOLED_BLOCKS
+#define NNIS_POOLED_BLOCKS 0
+#endif
+#if NNIS_POOLED_BLOCKS && !NNIS_SCORE_EXTRAS
+#error "pooled blocks come with the scores' extras"
+#endif
 
 struct AttnArgs {
   const void* q;  // [tokens, heads, HD]
@@ -78,7 +86,7 @@ struct AttnArgs {
   const float* bias;   // [heads, reach + 1]: added to the scaled score of a key `n` positions back, row min(n, reach)
   int reach;
   const float* sink;   // [heads]: a score that joins the softmax's denominator and has no value
-  // Pooled blocks beside a window (the row kernel only), off when `pool` is zero: entry b of a second set of pages
+  // Pooled blocks beside a window, off when `pool` is zero: entry b of a second set of pages
   // stands for the positions b * pool .. b * pool + pool - 1 and is seen by a query at position p, in the same
   // softmax as the window's keys, once the whole block has left the window: b * pool + pool - 1 <= p - window.
   const void* pool_k;
@@ -593,6 +601,12 @@ struct MfmaArgs {
   const float* bias;      // [heads, reach + 1], in the scores' own units (natural logarithm)
   int reach;
   const float* sink;      // [heads]
+  // with NNIS_POOLED_BLOCKS (see AttnArgs): off when `pool` is zero
+  const bf16_t* pool_k;
+  const bf16_t* pool_v;
+  const int* pool_table;  // [slots][pool_max_pages]
+  int pool_max_pages;
+  int pool;
 };
 
 __device__ __forceinline__ const bf16_t* k_page_ptr(const MfmaArgs& a, int page, int kv_head) {
@@ -816,6 +830,41 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
   }
 }
 
+#if NNIS_POOLED_BLOCKS
+// The pooled blocks that a wave's columns see, in the same softmax state as the window's keys: entry b of the
+// slot's pooled pages counts for a column whose window begins at lo once b * pool + pool - 1 < lo, i.e. b < lo / pool.
+// To the loops over key blocks the entries are keys 0 .. lo / pool - 1 of pages of their own, with no window, no
+// kept first keys and no bias.  The pages are dealt to `size` waves, this one their member `index`.
+template <int C, int RING>
+__device__ __forceinline__ void attend_pooled(AttnState<C>& st, const QFrag (&q)[C], const MfmaArgs& a, int slot, int kv_head,
+                                              int index, int size, const int (&lo)[C], const int (&hi)[C], int lane) {
+  int plo[C], phi[C];
+  int last = -1;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    plo[c] = 0;
+    phi[c] = hi[c] >= 0 ? lo[c] / a.pool - 1 : -1;
+    last = max(last, phi[c]);
+  }
+#pragma unroll
+  for (int offset = kWave / 2; offset > 0; offset >>= 1) last = max(last, __shfl_xor(last, offset, kWave));
+  if (last < 0) return;
+  MfmaArgs pa = a;
+  pa.k_pages = a.pool_k; pa.v_pages = a.pool_v; pa.max_pages = a.pool_max_pages; pa.bias = nullptr;
+  More<C> none;
+  none.reach = 0;
+  none.keep = 0;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    none.bias_row[c] = nullptr;
+    none.far_bias[c] = 0.0f;
+  }
+  const int page_count = last / kPageTokens + 1;
+  const int mine = page_count > index ? (page_count - index + size - 1) / size : 0;
+  attend_run<C, RING>(st, q, pa, a.pool_table + (size_t)slot * a.pool_max_pages, kv_head, index, size, mine, last, plo, phi, lane, none);
+}
+#endif
+
 // key blocks a prefilling wave has in flight: as many as its registers hold beside C columns' states.  Beyond 96
 // channels two columns and two blocks need more than 256 registers, which leaves a SIMD one wave: with one block
 // in flight two waves fit, and the other wave's work fills the wait (32/8 heads of 128, one wave an item, at 8,192
@@ -918,6 +967,9 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
 #endif
       const int mine = page_count > index ? (page_count - index + size - 1) / size : 0;  // pages of this wave
       attend_run<C, kPrefillRing<C>>(st, q, a, pages, kv_head, first_page + index, size, mine, last, lo, hi, lane, more);
+#if NNIS_POOLED_BLOCKS
+      if (a.pool > 0) attend_pooled<C, kPrefillRing<C>>(st, q, a, slot_of[which], kv_head, index, size, lo, hi, lane);
+#endif
     }
     if (!merge_group<C>(st, slots, index, size, rounds, lane)) return;
 #pragma unroll
@@ -1083,6 +1135,13 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(Mfma
 #endif
   const int mine = end > begin + wave ? (end - begin - wave + waves - 1) / waves : 0;  // pages of this wave
   attend_run<C, (kDecodeRing / C >= 2 ? kDecodeRing / C : 2)>(st, q, a, pages, kv_head, begin + wave, waves, mine, pos, lo, hi, lane, more);
+#if NNIS_POOLED_BLOCKS
+  // the pooled blocks go with the first run of the keys (with the step's tables the pooled pages are still the slot's)
+  if (a.pool > 0 && split == 0) {
+    const int pool_slot = a.rows_by_token ? a.tok_slot[token] : slot;
+    if (pool_slot >= 0) attend_pooled<C, (kDecodeRing / C >= 2 ? kDecodeRing / C : 2)>(st, q, a, pool_slot, kv_head, wave, waves, lo, hi, lane);
+  }
+#endif
   finish_decode<C>(st, live, a, merge, token, kv_head, split, wave, waves, lane);
 }
 
@@ -1422,6 +1481,18 @@ int fill_extras(MfmaArgs& a, int keep_first, const float* bias, int reach, const
                "attention: this module is compiled without kept first keys, a bias by distance and a sink");
   NNIS_REQUIRE(keep_first >= 0 && (bias == nullptr || reach >= 0), "attention: bad keep_first %d or reach %d", keep_first, reach);
   a.keep_first = a.window > 0 ? keep_first : 0; a.bias = bias; a.reach = reach; a.sink = sink;
+  a.pool_k = nullptr; a.pool_v = nullptr; a.pool_table = nullptr; a.pool_max_pages = 0; a.pool = 0;
+  return 0;
+}
+
+int fill_pooled(MfmaArgs& a, const void* pool_k, const void* pool_v, const int* pool_table, int pool_max_pages, int pool) {
+  NNIS_REQUIRE(pool >= 0, "attention: pooled blocks of %d tokens", pool);
+  if (pool == 0) return 0;
+  NNIS_REQUIRE(NNIS_POOLED_BLOCKS, "attention: this module is compiled without pooled blocks");
+  NNIS_REQUIRE(a.window > 0 && pool_k && pool_v && pool_table && pool_max_pages > 0,
+               "attention: pooled blocks (%d tokens each) need a window and pages of their own", pool);
+  a.pool_k = (const bf16_t*)pool_k; a.pool_v = (const bf16_t*)pool_v; a.pool_table = pool_table;
+  a.pool_max_pages = pool_max_pages; a.pool = pool;
   return 0;
 }
 }  // namespace
@@ -1470,15 +1541,18 @@ extern "C" int nnis_attention_prefill_max_waves(int heads, int kv_heads, int col
   return waves;
 }
 
-extern "C" int nnis_attention_prefill_bf16_more(const void* q, void* out, const void* k_pages, const void* v_pages,
-                                                const int* block_table, int max_pages, const int* tile_seq,
-                                                const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
-                                                const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
-                                                float scale, int waves, int columns, float softcap, int keep_first,
-                                                const float* bias, int reach, const float* sink, void* stream) {
+extern "C" int nnis_attention_prefill_bf16_pooled(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                                  const int* block_table, int max_pages, const int* tile_seq,
+                                                  const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
+                                                  const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
+                                                  float scale, int waves, int columns, float softcap, int keep_first,
+                                                  const float* bias, int reach, const float* sink, const void* pool_k,
+                                                  const void* pool_v, const int* pool_table, int pool_max_pages, int pool,
+                                                  void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale, softcap)) return 1;
   if (fill_extras(a, keep_first, bias, reach, sink)) return 1;
+  if (fill_pooled(a, pool_k, pool_v, pool_table, pool_max_pages, pool)) return 1;
   if (tiles <= 0) return 0;
   a.tile_seq = tile_seq; a.tile_row0 = tile_row0; a.seq_slot = seq_slot; a.seq_start = seq_start; a.seq_pos0 = seq_pos0;
   const int group = heads / kv_heads;
@@ -1553,15 +1627,17 @@ extern "C" int nnis_attention_decode_max_waves(int heads, int kv_heads) {
 // for columns or keys on lanes and fail where that kernel does not take the sizes.  combine: 0 leaves the
 // runs in `partial` ([tokens, heads, splits, head_dim + 4]: outputs, reference, sum) and writes no output: the
 // projection that follows, or nnis_attention_combine, adds them up.
-extern "C" int nnis_attention_decode_bf16_more(const void* q, void* out, const void* k_pages, const void* v_pages,
-                                               const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
-                                               int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
-                                               int splits, int waves, float* partial, int kind, int combine, int rows_by_token,
-                                               float softcap, int keep_first, const float* bias, int reach, const float* sink,
-                                               void* stream) {
+extern "C" int nnis_attention_decode_bf16_pooled(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                                 const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
+                                                 int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
+                                                 int splits, int waves, float* partial, int kind, int combine, int rows_by_token,
+                                                 float softcap, int keep_first, const float* bias, int reach, const float* sink,
+                                                 const void* pool_k, const void* pool_v, const int* pool_table, int pool_max_pages,
+                                                 int pool, void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale, softcap)) return 1;
   if (fill_extras(a, keep_first, bias, reach, sink)) return 1;
+  if (fill_pooled(a, pool_k, pool_v, pool_table, pool_max_pages, pool)) return 1;
   a.rows_by_token = rows_by_token ? 1 : 0;
   NNIS_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of splits %d", splits);
   NNIS_REQUIRE(splits == 1 || partial != nullptr, "attention: splits need scratch memory");
@@ -1617,6 +1693,28 @@ extern "C" int nnis_attention_decode_bf16_more(const void* q, void* out, const v
   return 0;
 }
 
+extern "C" int nnis_attention_decode_bf16_more(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                               const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
+                                               int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
+                                               int splits, int waves, float* partial, int kind, int combine, int rows_by_token,
+                                               float softcap, int keep_first, const float* bias, int reach, const float* sink,
+                                               void* stream) {
+  return nnis_attention_decode_bf16_pooled(q, out, k_pages, v_pages, block_table, max_pages, tok_slot, tok_pos, tokens, heads, kv_heads,
+                                           head_dim, window, scale, splits, waves, partial, kind, combine, rows_by_token, softcap,
+                                           keep_first, bias, reach, sink, nullptr, nullptr, nullptr, 0, 0, stream);
+}
+
+extern "C" int nnis_attention_prefill_bf16_more(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                                const int* block_table, int max_pages, const int* tile_seq,
+                                                const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
+                                                const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
+                                                float scale, int waves, int columns, float softcap, int keep_first,
+                                                const float* bias, int reach, const float* sink, void* stream) {
+  return nnis_attention_prefill_bf16_pooled(q, out, k_pages, v_pages, block_table, max_pages, tile_seq, tile_row0, tiles, seq_slot,
+                                            seq_start, seq_pos0, heads, kv_heads, head_dim, window, scale, waves, columns, softcap,
+                                            keep_first, bias, reach, sink, nullptr, nullptr, nullptr, 0, 0, stream);
+}
+
 extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
                                           const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
                                           int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
@@ -1654,6 +1752,16 @@ extern "C" int nnis_attention_prefill_tile_rows(int, int, int) { return 0; }
 extern "C" int nnis_attention_prefill_max_waves(int, int, int) { return 1; }
 extern "C" int nnis_attention_prefill_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
                                            int, const int*, const int*, const int*, int, int, int, int, float, int, int, float, void*) {
+  return nnis_fail("attention: the matrix-core kernels need keys and values in steps of 16 channels; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
+}
+extern "C" int nnis_attention_prefill_bf16_pooled(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
+                                                  int, const int*, const int*, const int*, int, int, int, int, float, int, int, float, int,
+                                                  const float*, int, const float*, const void*, const void*, const int*, int, int, void*) {
+  return nnis_fail("attention: the matrix-core kernels need keys and values in steps of 16 channels; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
+}
+extern "C" int nnis_attention_decode_bf16_pooled(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
+                                                 int, int, int, int, int, float, int, int, float*, int, int, int, float, int, const float*,
+                                                 int, const float*, const void*, const void*, const int*, int, int, void*) {
   return nnis_fail("attention: the matrix-core kernels need keys and values in steps of 16 channels; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
 }
 extern "C" int nnis_attention_prefill_bf16_more(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,

@@ -57,7 +57,7 @@ PREBUILT_WIDE_VALUES = ("attn_hd7v5c", "attn_hd32v16c", "attn_hd16v48c", "attn_h
                         # the sizes of the measurements of windowed and latent attention
                         "attn_hd64x", "attn_hd128x", "attn_hd160v128x", "attn_hd256v192x",
                         # capped scores with a sink: windows with pooled blocks
-                        "attn_hd16cx", "attn_hd32v16cx", "attn_hd24v40cx", "attn_hd64cx", "attn_hd128cx")
+                        "attn_hd16cxp", "attn_hd32v16cxp", "attn_hd24v40cx", "attn_hd24v40cxp", "attn_hd64cxp", "attn_hd128cxp", "attn_hd32xp")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -109,8 +109,12 @@ def register_module_family(prefix: str, recipe: Callable[[str], ModuleRecipe], r
 def _attention_recipe(rest: str) -> ModuleRecipe:
     """``attn_hd<N>``: keys and values of N channels; ``attn_hd<N>v<M>``: values of M; a ``c`` behind either: with a
     cap of the scores compiled in; an ``x`` at the very end: with the extras of the scores (first keys kept visible
-    beside a window, a bias by distance, a sink in the denominator) compiled into the matrix-core kernels."""
+    beside a window, a bias by distance, a sink in the denominator) compiled into the matrix-core kernels; ``xp``:
+    with pooled blocks beside a window as well."""
     name = rest
+    pooled = rest.endswith("xp")
+    if pooled:
+        rest = rest[:-1]
     extras = rest.endswith("x")
     if extras:
         rest = rest[:-1]
@@ -128,6 +132,8 @@ def _attention_recipe(rest: str) -> ModuleRecipe:
         defines.append(("NNIS_SCORE_CAP", "1"))
     if extras:
         defines.append(("NNIS_SCORE_EXTRAS", "1"))
+    if pooled:
+        defines.append(("NNIS_POOLED_BLOCKS", "1"))
     return ModuleRecipe(("attention.hip",), ("common.h",), tuple(defines), (("attention.hip", tuple(_VECTOR_SUMS)),))
 
 

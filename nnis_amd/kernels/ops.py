@@ -70,6 +70,12 @@ _ATTN_SIGNATURES = {
                                  _INT, _INT, _FLT, _INT, _FLT, _INT, _VOID, _INT, _VOID, _VOID],
     "nnis_attention_rows_pooled": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
                                    _INT, _INT, _FLT, _INT, _FLT, _INT, _VOID, _INT, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _VOID],
+    "nnis_attention_prefill_bf16_pooled": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
+                                           _INT, _INT, _INT, _FLT, _INT, _INT, _FLT, _INT, _VOID, _INT, _VOID,
+                                           _VOID, _VOID, _VOID, _INT, _INT, _VOID],
+    "nnis_attention_decode_bf16_pooled": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
+                                          _INT, _INT, _VOID, _INT, _INT, _INT, _FLT, _INT, _VOID, _INT, _VOID,
+                                          _VOID, _VOID, _VOID, _INT, _INT, _VOID],
     "nnis_attention_prefill_tile_rows": [_INT, _INT, _INT],
     "nnis_attention_prefill_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
                                     _INT, _INT, _INT, _FLT, _INT, _INT, _FLT, _VOID],
@@ -224,15 +230,17 @@ def attention_check(head_dim: int, value_dim: Optional[int] = None, most: int = 
         _wide_heads.add((head_dim, value_dim or head_dim))
 
 
-def attention_module_name(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None) -> str:
+def attention_module_name(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None, pooled=None) -> str:
     """The module compiled for keys of ``head_dim`` channels and values of ``value_dim`` (None: as the keys), with a
-    cap of the scores (``softcap`` > 0) or without, and with the scores' extras (``ScoreExtras``) or without."""
+    cap of the scores (``softcap`` > 0) or without, with the scores' extras (``ScoreExtras``) or without, and, with the
+    extras, with pooled blocks beside a window (``PooledBlocks``) or without."""
     wide = value_dim is not None and value_dim != head_dim
-    return (f"attn_hd{head_dim}v{value_dim}" if wide else f"attn_hd{head_dim}") + ("c" if softcap else "") + ("x" if extras else "")
+    return ((f"attn_hd{head_dim}v{value_dim}" if wide else f"attn_hd{head_dim}") + ("c" if softcap else "")
+            + ("xp" if pooled is not None else ("x" if extras else "")))
 
 
-def attention_module(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None):
-    name = attention_module_name(head_dim, value_dim, softcap, extras)
+def attention_module(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None, pooled=None):
+    name = attention_module_name(head_dim, value_dim, softcap, extras, pooled)
     if name not in _attn:
         accepted = (head_dim, value_dim or head_dim) in _wide_heads
         attention_check(head_dim, value_dim, ATTENTION_ROWS_MOST_CHANNELS if accepted else ATTENTION_MOST_CHANNELS)
@@ -565,7 +573,7 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_
         raise KernelError("attention: key and value pages differ in type")
     if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or block_table.dtype != torch.int32:
         raise KernelError("attention: tok_slot, tok_pos and block_table must be int32")
-    lib = attention_module(head_dim, value_dim, softcap, extras)
+    lib = attention_module(head_dim, value_dim, softcap, extras, pooled)
     if pooled is not None:
         extras = extras or ScoreExtras()
         extras.check(heads)
@@ -971,20 +979,20 @@ def _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_di
             raise KernelError(f"attention: the matrix-core kernels take bfloat16, {what} is {t.dtype}")
 
 
-def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0, extras=None) -> int:
+def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0, extras=None, pooled=None) -> int:
     """Query rows per work item of ``attention_prefill_bf16`` for these sizes.
     ``columns``: the most 16-column tiles (query tiles x heads of a group) a
     wave carries; 0 for as many as the head size allows."""
-    return attention_module(head_dim, value_dim, softcap, extras).nnis_attention_prefill_tile_rows(heads, kv_heads, columns)
+    return attention_module(head_dim, value_dim, softcap, extras, pooled).nnis_attention_prefill_tile_rows(heads, kv_heads, columns)
 
 
-def prefill_max_waves(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0, extras=None) -> int:
-    return attention_module(head_dim, value_dim, softcap, extras).nnis_attention_prefill_max_waves(heads, kv_heads, columns)
+def prefill_max_waves(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0, extras=None, pooled=None) -> int:
+    return attention_module(head_dim, value_dim, softcap, extras, pooled).nnis_attention_prefill_max_waves(heads, kv_heads, columns)
 
 
 def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile_row0, seq_slot, seq_start, seq_pos0,
                            heads, kv_heads, head_dim, scale, window=0, waves=1, columns=0, value_dim=None, softcap=0.0,
-                           extras: Optional[ScoreExtras] = None):
+                           extras: Optional[ScoreExtras] = None, pooled: Optional[PooledBlocks] = None):
     """Causal attention of whole runs of new tokens over the cache, on the
     matrix cores.  ``tile_seq``/``tile_row0`` (int32) name, per work item, a
     sequence of the step and the first of ``prefill_tile_rows`` rows of its
@@ -997,7 +1005,18 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
     tiles = tile_seq.numel()
     if tile_row0.numel() != tiles or seq_start.numel() != seq_slot.numel() + 1 or seq_pos0.numel() != seq_slot.numel():
         raise KernelError("attention: step metadata arrays do not fit each other")
-    lib = attention_module(head_dim, value_dim, softcap, extras)
+    lib = attention_module(head_dim, value_dim, softcap, extras, pooled)
+    if pooled is not None:
+        extras = extras or ScoreExtras()
+        extras.check(heads)
+        pooled.check(k_pages, v_pages, kv_heads, head_dim, value_dim or head_dim, window)
+        _check(lib, lib.nnis_attention_prefill_bf16_pooled(
+            q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+            tile_seq.data_ptr(), tile_row0.data_ptr(), tiles, seq_slot.data_ptr(), seq_start.data_ptr(), seq_pos0.data_ptr(), heads,
+            kv_heads, head_dim, int(window), float(scale), int(waves), int(columns), float(softcap), extras.keep_first,
+            _ptr(extras.bias), extras.reach, _ptr(extras.sink), pooled.k_pages.data_ptr(), pooled.v_pages.data_ptr(),
+            pooled.block_table.data_ptr(), pooled.block_table.shape[1], pooled.pool, _stream()))
+        return out
     if extras:
         extras.check(heads)
         _check(lib, lib.nnis_attention_prefill_bf16_more(
@@ -1016,7 +1035,7 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
 
 def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_pos, heads, kv_heads, head_dim, scale,
                           window=0, splits=1, partial=None, waves=1, kernel="auto", keep_runs=False, token_pages=None,
-                          value_dim=None, softcap=0.0, extras: Optional[ScoreExtras] = None):
+                          value_dim=None, softcap=0.0, extras: Optional[ScoreExtras] = None, pooled: Optional[PooledBlocks] = None):
     """One query token per sequence over its cached keys.  The keys are cut
     into ``splits`` runs, each a block of ``waves`` waves that deal its pages
     among themselves and merge in LDS; the runs are summed by a second kernel.
@@ -1047,8 +1066,19 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
         if partial is None or partial.dtype != torch.float32 or partial.numel() < tokens * heads * splits * (value_dim + 4):
             raise KernelError("attention: splits need float32 scratch of tokens * heads * splits * (value channels + 4)")
         _dev(partial, "partial")
-    lib = attention_module(head_dim, value_dim, softcap, extras)
-    if extras:
+    lib = attention_module(head_dim, value_dim, softcap, extras, pooled)
+    if pooled is not None:
+        extras = extras or ScoreExtras()
+        extras.check(heads)
+        pooled.check(k_pages, v_pages, kv_heads, head_dim, value_dim, window)
+        _check(lib, lib.nnis_attention_decode_bf16_pooled(
+            q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), table.shape[1],
+            tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window), float(scale), int(splits),
+            int(waves), _ptr(partial) if splits > 1 else None, _DECODE_KERNELS["columns"], 0 if (keep_runs and splits > 1) else 1,
+            1 if token_pages is not None else 0, float(softcap), extras.keep_first, _ptr(extras.bias), extras.reach,
+            _ptr(extras.sink), pooled.k_pages.data_ptr(), pooled.v_pages.data_ptr(), pooled.block_table.data_ptr(),
+            pooled.block_table.shape[1], pooled.pool, _stream()))
+    elif extras:
         extras.check(heads)
         _check(lib, lib.nnis_attention_decode_bf16_more(
             q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), table.shape[1],
@@ -1128,8 +1158,8 @@ def decode_scratch_held(device):
     return _decode_scratch.get((device.type, device.index))
 
 
-def decode_max_waves(heads: int, kv_heads: int, head_dim: int, value_dim=None, softcap=0.0, extras=None) -> int:
-    return attention_module(head_dim, value_dim, softcap, extras).nnis_attention_decode_max_waves(heads, kv_heads)
+def decode_max_waves(heads: int, kv_heads: int, head_dim: int, value_dim=None, softcap=0.0, extras=None, pooled=None) -> int:
+    return attention_module(head_dim, value_dim, softcap, extras, pooled).nnis_attention_decode_max_waves(heads, kv_heads)
 
 
 def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4, width: int = 0):
@@ -1295,11 +1325,11 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     (waves, columns) of a step of prompts (``prefill_plan``); None: as those
     functions choose for the step's planned sizes."""
     value_dim = value_dim or head_dim
-    fast = pooled is None and attention_on_matrix_cores(q.dtype, view.k_pages.dtype, head_dim, value_dim, softcap, extras)
+    fast = attention_on_matrix_cores(q.dtype, view.k_pages.dtype, head_dim, value_dim, softcap, extras)
     size = max(head_dim, value_dim)  # what a wave's registers are sized by
     if fast and ctx.decode and heads // kv_heads <= 16 * (4 if size <= 64 else (2 if size <= 128 else 1)):
         splits, waves = plan or decode_plan(ctx.batch, kv_heads, ctx.planned_len, width=heads * value_dim)
-        waves = min(waves, decode_max_waves(heads, kv_heads, head_dim, value_dim, softcap, extras))
+        waves = min(waves, decode_max_waves(heads, kv_heads, head_dim, value_dim, softcap, extras, pooled))
         partial = None
         if splits > 1:
             partial = decode_scratch(q.device, q.shape[0] * heads * splits * (value_dim + 4))
@@ -1307,17 +1337,17 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
                                      kv_heads, head_dim, scale, window, splits, partial, waves,
                                      keep_runs=keep_runs and q.shape[0] <= KEY_RUNS_MOST_TOKENS,
                                      token_pages=tables.pages if tables is not None else None, value_dim=value_dim, softcap=softcap,
-                                     extras=extras)
+                                     extras=extras, pooled=pooled)
     if fast and not ctx.decode:
         # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
         # a block deal the keys among themselves (their merge lives in LDS).
         waves, columns = plan or prefill_plan(ctx.planned_len, ctx.planned_rows, heads, size, kv_heads)
-        waves = min(waves, prefill_max_waves(heads, kv_heads, head_dim, columns, value_dim, softcap, extras))
-        rows = prefill_tile_rows(heads, kv_heads, head_dim, columns, value_dim, softcap, extras)
+        waves = min(waves, prefill_max_waves(heads, kv_heads, head_dim, columns, value_dim, softcap, extras, pooled))
+        rows = prefill_tile_rows(heads, kv_heads, head_dim, columns, value_dim, softcap, extras, pooled)
         tiles = ctx.lists.device_list(("attention_tiles", rows), lambda new, first, padded: prefill_tile_list(new, first, padded, rows))
         return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tiles[0], tiles[1],
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,
-                                      waves, columns, value_dim, softcap, extras)
+                                      waves, columns, value_dim, softcap, extras, pooled)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                           kv_heads, head_dim, scale, window, value_dim, softcap, extras, pooled)
 

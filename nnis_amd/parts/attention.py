@@ -325,14 +325,13 @@ class GatedWindowAttention(Mixer):
         return self._pooled_request()
 
     def check(self, rt):
-        # (pooled blocks take the row kernel, which carries heads beyond the matrix-core kernels' sizes too)
         rt.ops.attention_check(self.head_dim, self.value_dim)
         rot_dim = getattr(self.position, "rot_dim", 0)
         if rot_dim > self.head_dim:
             raise InvalidInput(f"a rotation of {rot_dim} channels does not fit heads of {self.head_dim}")
 
     def _matrix_cores(self, rt) -> bool:
-        return not self.pool and rt.ops.attention_on_matrix_cores(rt.dtype, rt.dtype, self.head_dim, self.value_dim, self.softcap, self.extras)
+        return rt.ops.attention_on_matrix_cores(rt.dtype, rt.dtype, self.head_dim, self.value_dim, self.softcap, self.extras)
 
     def decode_plan(self, batch, longest, rt):
         if not self._matrix_cores(rt):

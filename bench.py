@@ -39,6 +39,12 @@ window with kept first tokens, a bias by distance and a sink; attention over a
 cached latent, plain and with a rotated part, a sink and gates; norms without
 statistics before and after every sublayer).
 
+``--workload robopel`` measures the Robopel design (attention with normed and
+rotated heads, a window with pooled blocks, a sink and gated heads, some layers
+reading an earlier layer's keys; minGRU; PolyNorm and routed feed-forwards;
+norms on the sublayers' outputs only) beside a Mutedra of windowed-attention
+layers of the same width, layers, heads, window, inner size and vocabulary.
+
 Peaks used for the fractions are the published MI355X ones: HBM 8 TB/s; dense
 matrix rate 2.5 PFLOP/s for bfloat16, 157.3 TFLOP/s for 32-bit.
 """
@@ -220,7 +226,7 @@ def prefill_run(shape, rng, tokens=2048):
     del engine
     torch.cuda.empty_cache()
     seconds = sorted(times[3:])[3]  # the median of seven runs of a shape that has come before (and is captured, where it is)
-    flops = {"Zifunex": zifunex_step_flops, "Mutedra": mutedra_step_flops}.get(shape.config.get("architecture"), step_flops)(
+    flops = {"Zifunex": zifunex_step_flops, "Mutedra": mutedra_step_flops, "Robopel": robopel_step_flops}.get(shape.config.get("architecture"), step_flops)(
         shape.config, [tokens], 1)
     return {"value": round(tokens / seconds, 1), "tokens": tokens, "ms": round(1000.0 * seconds, 3),
             "frac": round(flops / seconds / FLOP_PEAK[shape.dtype], 5), "first_ms": round(1000.0 * times[0], 3)}
@@ -381,13 +387,80 @@ def mutedra_twin_config(sizes):
                   max_position_embeddings=ZIFUNEX_CONTEXT, tie_word_embeddings=False)
 
 
-def design_run(args, rng, design, sets, config_of, twin_of):
+# Robopel at two sets of layer sizes: A = attention with keys of its own and a PolyNorm feed-forward, K = attention that
+# reads the keys of the A before it, G = minGRU with a routed feed-forward (experts, chosen, identity outputs, inner
+# size of an expert).  Windows with pooled blocks of 64 tokens; a bent rotation of the whole head.
+ROBOPEL_SETS = {
+    "w1024": dict(width=1024, ff=2816, attention=(16, 4, 64, 64), window=(512, 64), gru=1024, moe=(8, 2, 1, 704)),
+    "w2048": dict(width=2048, ff=5632, attention=(16, 4, 128, 128), window=(1024, 64), gru=2048, moe=(8, 2, 1, 1408)),
+}
+ROBOPEL_LAYERS = "AGKGAGKG"
+
+
+def robopel_config(sizes):
+    heads, kv_heads, dim, vdim = sizes["attention"]
+    experts, top, identity, expert_ff = sizes["moe"]
+    layers, owner = [], None
+    for index, kind in enumerate(ROBOPEL_LAYERS):
+        if kind == "G":
+            layers.append({"type": "mingru", "mixer": {"width": sizes["gru"]}, "mlp": {
+                "kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "identity": identity}}})
+            continue
+        mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "softcap": 30.0,
+                 "rot": {"dims": dim, "base": 10000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048}},
+                 "mask": {"size": sizes["window"][0], "pool": sizes["window"][1]}}
+        if kind == "K":
+            mixer["kv_from"] = owner
+        else:
+            owner = index
+        layers.append({"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": sizes["ff"]}})
+    return {"architecture": "Robopel", "vocab": ZIFUNEX_VOCAB, "width": sizes["width"], "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+            "layers": layers}
+
+
+def robopel_step_flops(config, tokens_per_sequence, wanted_rows):
+    """Multiply-adds x2 of one step over whole prompts from empty slots: the projections, a window's keys and the
+    pooled blocks before it, and of the experts those that a token has chosen (the library multiplies all of them)."""
+    w = config["width"]
+    total = 0
+    for n in tokens_per_sequence:
+        for layer in config["layers"]:
+            m = layer["mixer"]
+            if layer["type"] == "attention":
+                own = 0 if m.get("kv_from") is not None else m["kv_heads"] * (m["dim"] + m["vdim"])
+                per_token = (m["heads"] * m["dim"] + own + 2 * m["heads"] * m["vdim"]) * w
+                size, pool = m["mask"]["size"], m["mask"]["pool"]
+                keys = sum(min(i + 1, size) + max(0, i + 1 - size) // pool for i in range(n))
+                total += 2 * per_token * n + 2 * m["heads"] * (m["dim"] + m["vdim"]) * keys
+            else:
+                total += 2 * 4 * m["width"] * w * n
+            mlp = layer["mlp"]
+            if mlp is not None and mlp["kind"] == "dense":
+                total += 2 * 2 * w * mlp["ff"] * n
+            elif mlp is not None:
+                router = mlp["router"]
+                total += 2 * (2 * w * mlp["expert"]["ff"] * router["top"] + (router["experts"] + router["identity"]) * w) * n
+    return total + 2 * wanted_rows * w * config["vocab"]
+
+
+def robopel_twin_config(sizes):
+    """The closest model the library had: a Mutedra of windowed-attention layers (a sink, kept first tokens, a bias by
+    distance) with gated feed-forwards, of the same width, layers, heads, window, inner size and vocabulary."""
+    heads, kv_heads, dim, vdim = sizes["attention"]
+    layer = {"type": "attention", "mlp": {"kind": "dense", "ff": sizes["ff"]}, "mixer": {
+        "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "bias_max": 128, "bias_buckets": 32,
+        "mask": {"size": sizes["window"][0], "keep_first": 4}}}
+    return {"architecture": "Mutedra", "vocab": ZIFUNEX_VOCAB, "width": sizes["width"], "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+            "logit_softcap": 30.0, "layers": [layer] * len(ROBOPEL_LAYERS), "loop": {"start": 0, "stop": len(ROBOPEL_LAYERS), "times": 1}}
+
+
+def design_run(args, rng, design, sets, config_of, twin_of, twin="llama"):
     """Each set of sizes: the design's model and its Llama twin, a prompt of 2,048 tokens and decode at batch 1, 8, 64."""
     import torch
 
     out = {}
     for name, sizes in sets.items():
-        for which, config in ((design, config_of(sizes)), ("llama", twin_of(sizes))):
+        for which, config in ((design, config_of(sizes)), (twin, twin_of(sizes))):
             torch.cuda.empty_cache()
             with tempfile.TemporaryDirectory() as folder:
                 shape = Shape(f"{which}-{name}", 0, args.dtype, args.seed, folder, config=config, context=ZIFUNEX_CONTEXT)
@@ -433,7 +506,7 @@ def main() -> int:
     parser.add_argument("--no-other-shapes", action="store_true", help="points of the headline's shape only")
     parser.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the decode batches")
     parser.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the decode batches (within the context)")
-    parser.add_argument("--workload", choices=["tinyllama-ragged", "zifunex", "mutedra"], help="run this workload alone")
+    parser.add_argument("--workload", choices=["tinyllama-ragged", "zifunex", "mutedra", "robopel"], help="run this workload alone")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -463,6 +536,18 @@ def main() -> int:
             "ms_per_step": head["ms_per_step"], "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic: random weights from a seed, uniform-random token ids",
             "config": {"model": "Mutedra, 8 layers of width 2048 (decode at batch 8)", "sets": MUTEDRA_SETS, "layers": MUTEDRA_LAYERS,
+                       "vocab": ZIFUNEX_VOCAB, "context": ZIFUNEX_CONTEXT, "prompt_min": args.prompt_min, "prompt_max": args.prompt_max},
+            "models": models, "env": environment()}))
+        return 0
+    if args.workload == "robopel":
+        models = design_run(args, rng, "robopel", ROBOPEL_SETS, robopel_config, robopel_twin_config, twin="mutedra")
+        head = models["robopel-w2048"]["decode_b8"]
+        print(json.dumps({
+            "metric": "Robopel at two sets of layer sizes beside a Mutedra of windowed attention of the same sizes: prefill of 2,048 tokens, decode at batch 1, 8, 64",
+            "value": head["tokens_per_second"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": head["ms_per_step"], "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic: random weights from a seed, uniform-random token ids",
+            "config": {"model": "Robopel, 8 layers of width 2048 (decode at batch 8)", "sets": ROBOPEL_SETS, "layers": ROBOPEL_LAYERS,
                        "vocab": ZIFUNEX_VOCAB, "context": ZIFUNEX_CONTEXT, "prompt_min": args.prompt_min, "prompt_max": args.prompt_max},
             "models": models, "env": environment()}))
         return 0

@@ -56,8 +56,11 @@ PREBUILT_WIDE_VALUES = ("attn_hd7v5c", "attn_hd32v16c", "attn_hd16v48c", "attn_h
                         "attn_hd32v16x", "attn_hd16v48x", "attn_hd48v32x", "attn_hd96v64x", "attn_hd32v24x", "attn_hd40", "attn_hd288v272x", "attn_hd16x",
                         # the sizes of the measurements of windowed and latent attention
                         "attn_hd64x", "attn_hd128x", "attn_hd160v128x", "attn_hd256v192x",
-                        # capped scores with a sink: windows with pooled blocks
-                        "attn_hd16cxp", "attn_hd32v16cxp", "attn_hd24v40cx", "attn_hd24v40cxp", "attn_hd64cxp", "attn_hd128cxp", "attn_hd32xp")
+                        # a sink with and without a cap, windows with and without pooled blocks: what the tests use, and the
+                        # sizes of the measurements
+                        "attn_hd32v16cx", "attn_hd32v16xp", "attn_hd32v16cxp", "attn_hd16v48cx", "attn_hd16v48xp", "attn_hd16v48cxp",
+                        "attn_hd24v40x", "attn_hd24v40cx", "attn_hd24v40xp", "attn_hd24v40cxp", "attn_hd16cx", "attn_hd16xp", "attn_hd16cxp",
+                        "attn_hd20v12xp", "attn_hd32xp", "attn_hd64cxp", "attn_hd128cxp")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

@@ -187,23 +187,19 @@ def _sub(weights, prefix):
 
 
 class PlainRobopel:
-    """The whole model over one sequence from its first token.  ``weights``: checkpoint names -> 64-bit tensors."""
+    """The whole model over one sequence from its first token, from a folder with config.json and model.safetensors."""
 
-    def __init__(self, config, weights, rnd=identity):
-        self.config, self.rnd = config, rnd
-        self.w = {name: (value.double() if value.is_floating_point() else value) for name, value in weights.items()}
-
-    @classmethod
-    def from_folder(cls, folder, rnd=identity):
+    def __init__(self, folder):
         with open(os.path.join(folder, "config.json")) as handle:
-            config = json.load(handle)
-        return cls(config, load_file(os.path.join(folder, "model.safetensors")), rnd)
+            self.config = json.load(handle)
+        self.w = {name: (value.double() if value.is_floating_point() else value)
+                  for name, value in load_file(os.path.join(folder, "model.safetensors")).items()}
 
-    def forward(self, tokens, layers_out=None):
-        """Logits [tokens, vocab]; ``layers_out`` (a list) gets the stream after every layer."""
-        cfg, w, rnd = self.config, self.w, self.rnd
+    def logits(self, ids, rnd=identity, stream_after=None):
+        """Logits [tokens, vocab]; ``stream_after`` (a list) gets the stream after every layer."""
+        cfg, w = self.config, self.w
         eps = cfg["norm"]["eps"]
-        x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * cfg.get("embedding", {}).get("scale", 1.0)
+        x = w["embed"][torch.as_tensor(list(ids), dtype=torch.long)] * (cfg.get("embedding") or {}).get("scale", 1.0)
         caches = {}
         for index, layer in enumerate(cfg["layers"]):
             prefix = f"l{index}."
@@ -223,6 +219,13 @@ class PlainRobopel:
                 else:
                     y, _ = routed_feed_forward(h, _sub(w, prefix + "mlp."), mlp["router"], rnd)
                 x = x + rms_norm(y, 1.0 + w[prefix + "norm2"], eps)
-            if layers_out is not None:
-                layers_out.append(x.clone())
+            if stream_after is not None:
+                stream_after.append(x.clone())
         return rms_norm(x, 1.0 + w["final.norm"], eps) @ w["head"].T
+
+    def greedy(self, ids, count):
+        ids, out = list(ids), []
+        for _ in range(count):
+            out.append(int(self.logits(ids)[-1].argmax()))
+            ids.append(out[-1])
+        return out

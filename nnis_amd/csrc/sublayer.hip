@@ -4,6 +4,7 @@
 //   cast_rows          rows of one type as rows of another (the 32-bit stream as a sublayer's input)
 //   rms_post_step      x += y / rms(y) * (offset + w), and the stream's rows in the activation type
 //   poly_norm          a N(z) + b N(z^2) + c N(z^3) + e, N a division by the root mean square of a row
+//   router_logits      a router's logits as 32-bit dot products
 //   route_top          softmax of router logits, the `top` largest of score + correction, dense weights out
 //   routed_act         weight[row, expert] * relu(z)^2 on the experts' fused up projection
 //   rows_axpy          y[row] += c[row] * h[row]
@@ -26,18 +27,42 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf
 // in place in the 32-bit stream, and h[row] = the new x in the activation type (what the next sublayer reads).
 // A block a row; the row is read twice (the second time from the caches).
 // -----------------------------------------------------------------------------
+constexpr int kPostKeep = 16;  // values of a row that a thread keeps in registers between the two passes
+
 __global__ __launch_bounds__(256) void rms_post_step_kernel(float* __restrict__ x, const void* __restrict__ y, int y_dtype,
                                                             const void* __restrict__ weight, int w_dtype, float offset, float eps,
                                                             void* __restrict__ h, int h_dtype, int width) {
   __shared__ float scratch[16];
   const size_t base = (size_t)blockIdx.x * width;
+  // everything the row needs is asked for before the sum is waited for: y, the stream and the weight, up to
+  // kPostKeep values a thread; what lies beyond (rows wider than kPostKeep x the block) is read a second time
+  float ys[kPostKeep], xs[kPostKeep], ws[kPostKeep];
   float ss = 0.0f;
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+#pragma unroll
+  for (int i = 0; i < kPostKeep; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    if (c < width) {
+      ys[i] = load_as_f32(y, y_dtype, base + c);
+      xs[i] = x[base + c];
+      ws[i] = offset + load_as_f32(weight, w_dtype, c);
+      ss = fmaf(ys[i], ys[i], ss);
+    }
+  }
+  for (int c = threadIdx.x + kPostKeep * blockDim.x; c < width; c += blockDim.x) {
     const float v = load_as_f32(y, y_dtype, base + c);
     ss = fmaf(v, v, ss);
   }
   const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+#pragma unroll
+  for (int i = 0; i < kPostKeep; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    if (c < width) {
+      const float sum = xs[i] + ys[i] * inv * ws[i];
+      x[base + c] = sum;
+      if (h) store_from_f32(h, h_dtype, base + c, sum);
+    }
+  }
+  for (int c = threadIdx.x + kPostKeep * blockDim.x; c < width; c += blockDim.x) {
     const float v = load_as_f32(y, y_dtype, base + c);
     const float sum = x[base + c] + v * inv * (offset + load_as_f32(weight, w_dtype, c));
     x[base + c] = sum;
@@ -49,26 +74,76 @@ __global__ __launch_bounds__(256) void rms_post_step_kernel(float* __restrict__ 
 // PolyNorm: out = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e, powers element by element, each root mean
 // square over the row with eps inside the root; coef = (a, b, c, e) in device memory.
 // -----------------------------------------------------------------------------
+constexpr int kPolyKeep = 32;  // values of a row that a thread keeps in registers between the two passes
+
 __global__ __launch_bounds__(256) void poly_norm_kernel(const void* __restrict__ z, int z_dtype, const float* __restrict__ coef,
                                                         float eps, void* __restrict__ out, int out_dtype, int width) {
   __shared__ float scratch[3][16];
   const size_t base = (size_t)blockIdx.x * width;
+  float zs[kPolyKeep];
   float s2 = 0.0f, s4 = 0.0f, s6 = 0.0f;
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
-    const float v = load_as_f32(z, z_dtype, base + c);
+  auto add = [&](float v) {
     const float v2 = v * v;
     s2 += v2;
     s4 = fmaf(v2, v2, s4);
     s6 = fmaf(v2 * v, v2 * v, s6);
+  };
+#pragma unroll
+  for (int i = 0; i < kPolyKeep; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    if (c < width) {
+      zs[i] = load_as_f32(z, z_dtype, base + c);
+      add(zs[i]);
+    }
   }
+  for (int c = threadIdx.x + kPolyKeep * blockDim.x; c < width; c += blockDim.x) add(load_as_f32(z, z_dtype, base + c));
   const float n = (float)width;
   const float i1 = 1.0f / sqrtf(block_sum(s2, scratch[0]) / n + eps);
   const float i2 = 1.0f / sqrtf(block_sum(s4, scratch[1]) / n + eps);
   const float i3 = 1.0f / sqrtf(block_sum(s6, scratch[2]) / n + eps);
   const float a = coef[0] * i1, b = coef[1] * i2, cc = coef[2] * i3, e = coef[3];
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+#pragma unroll
+  for (int i = 0; i < kPolyKeep; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    if (c < width) store_from_f32(out, out_dtype, base + c, fmaf(zs[i], fmaf(zs[i], fmaf(zs[i], cc, b), a), e));
+  }
+  for (int c = threadIdx.x + kPolyKeep * blockDim.x; c < width; c += blockDim.x) {
     const float v = load_as_f32(z, z_dtype, base + c);
     store_from_f32(out, out_dtype, base + c, fmaf(v, fmaf(v, fmaf(v, cc, b), a), e));
+  }
+}
+
+// -----------------------------------------------------------------------------
+// A router's logits: logits[row, e] = sum_c x[row, c] * w[e, c] in 32-bit, w float32 [n, width].  A block takes R rows,
+// kept in LDS as floats; a wave takes an output at a time for all of them (lanes stride over the channels), so a row
+// of the weight is read once a block.
+// -----------------------------------------------------------------------------
+template <int R>
+__global__ __launch_bounds__(256) void router_logits_kernel(const void* __restrict__ x, int x_dtype, const float* __restrict__ w,
+                                                            float* __restrict__ logits, int rows, int n, int width) {
+  extern __shared__ float xs[];  // [R][width]
+  const int row0 = blockIdx.x * R;
+  for (int i = threadIdx.x; i < R * width; i += blockDim.x) {
+    const int r = i / width;
+    xs[i] = row0 + r < rows ? load_as_f32(x, x_dtype, (size_t)(row0 + r) * width + i % width) : 0.0f;
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, waves = blockDim.x / kWave;
+  for (int e = wave; e < n; e += waves) {
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+    const float* row = w + (size_t)e * width;
+    for (int c = lane; c < width; c += kWave) {
+      const float wv = row[c];
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] = fmaf(xs[r * width + c], wv, acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float total = wave_sum(acc[r]);
+      if (lane == 0 && row0 + r < rows) logits[(size_t)(row0 + r) * n + e] = total;
+    }
   }
 }
 
@@ -158,6 +233,26 @@ __global__ void routed_act_kernel(const void* __restrict__ z, int z_dtype, const
   const float g = gates[row * experts + e];
   const float v = fmaxf(load_as_f32(z, z_dtype, i), 0.0f);
   store_from_f32(out, out_dtype, i, g == 0.0f ? 0.0f : g * v * v);
+}
+
+// the same, eight bfloat16 values a thread (ff a multiple of 8)
+__global__ void routed_act_bf16x8_kernel(const bf16_t* __restrict__ z, const float* __restrict__ gates, bf16_t* __restrict__ out,
+                                         int experts, int ff8, size_t total8) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  const size_t per_row = (size_t)experts * ff8;
+  const size_t row = i / per_row;
+  const int e = (int)((i % per_row) / ff8);
+  const float g = gates[row * experts + e];
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+  bf16x8_t v = g == 0.0f ? bf16x8_t{} : *(const bf16x8_t*)(z + i * 8);
+  bf16x8_t o;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const float a = fmaxf((float)v[k], 0.0f);
+    o[k] = (__bf16)(g == 0.0f ? 0.0f : g * a * a);
+  }
+  *(bf16x8_t*)(out + i * 8) = o;
 }
 
 // y[row, c] += keep[row] * h[row, c]
@@ -291,7 +386,10 @@ struct PoolArgs {
   int kv_heads, head_dim, value_dim, pool;
 };
 
-__global__ __launch_bounds__(128) void pool_blocks_kernel(PoolArgs a) {
+constexpr int kPoolMostChannels = 2048;  // key and value channels of a head together
+
+__global__ __launch_bounds__(256) void pool_blocks_kernel(PoolArgs a) {
+  __shared__ float part[4][kPoolMostChannels];
   const int token = blockIdx.x;
   const int kv_head = blockIdx.y;
   const int slot = a.tok_slot[token];
@@ -305,16 +403,25 @@ __global__ __launch_bounds__(128) void pool_blocks_kernel(PoolArgs a) {
   const int out_at = b % kPageTokens;
   const float share = 1.0f / (float)a.pool;
   const int hd = a.head_dim, vd = a.value_dim;
-  for (int d = threadIdx.x; d < hd + vd; d += blockDim.x) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  // the block's tokens are dealt to the four waves; a wave's lanes take the channels
+  for (int d = lane; d < hd + vd; d += kWave) {
     const bool key = d < hd;
     const int c = key ? d : d - hd;
     float sum = 0.0f;
-    for (int j = 0; j < a.pool; ++j) {
+    for (int j = wave; j < a.pool; j += 4) {
       const int p = first + j;
       const size_t page = (size_t)pages[p / kPageTokens] * a.kv_heads + kv_head;
       sum += key ? load_as_f32(a.k_pages, a.cache_dtype, page * nnis_k_page_elems(hd) + nnis_k_offset(p % kPageTokens, c))
                  : load_as_f32(a.v_pages, a.cache_dtype, page * nnis_v_page_elems(vd) + nnis_v_offset(c, p % kPageTokens));
     }
+    part[wave][d] = sum;
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < hd + vd; d += blockDim.x) {
+    const bool key = d < hd;
+    const int c = key ? d : d - hd;
+    const float sum = (part[0][d] + part[1][d]) + (part[2][d] + part[3][d]);
     const size_t out = (size_t)out_page * a.kv_heads + kv_head;
     if (key) {
       store_from_f32(a.pool_k, a.cache_dtype, out * nnis_k_page_elems(hd) + nnis_k_offset(out_at, c), sum * share);
@@ -371,6 +478,26 @@ extern "C" int nnis_poly_norm(const void* z, int z_dtype, const float* coef, flo
   return 0;
 }
 
+extern "C" int nnis_router_logits(const void* x, int x_dtype, const float* w, float* logits, int rows, int n, int width, void* stream) {
+  NNIS_REQUIRE(x && w && logits && n > 0 && width > 0, "router_logits: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(x_dtype), "router_logits: unknown dtype");
+  NNIS_REQUIRE(width <= 16384, "router_logits: rows of up to 16384 channels, got %d", width);
+  if (rows <= 0) return 0;
+  // several rows a block where they fit 48 KB of LDS and there are rows enough to fill the chip with such blocks
+  const int together = rows <= 256 ? 1 : (width <= 3072 ? 4 : (width <= 6144 ? 2 : 1));
+  const size_t lds = (size_t)together * width * sizeof(float);
+  const dim3 grid((rows + together - 1) / together);
+  if (together == 4) {
+    hipLaunchKernelGGL((router_logits_kernel<4>), grid, dim3(256), lds, (hipStream_t)stream, x, x_dtype, w, logits, rows, n, width);
+  } else if (together == 2) {
+    hipLaunchKernelGGL((router_logits_kernel<2>), grid, dim3(256), lds, (hipStream_t)stream, x, x_dtype, w, logits, rows, n, width);
+  } else {
+    hipLaunchKernelGGL((router_logits_kernel<1>), grid, dim3(256), lds, (hipStream_t)stream, x, x_dtype, w, logits, rows, n, width);
+  }
+  NNIS_LAUNCH_CHECK("router_logits");
+  return 0;
+}
+
 extern "C" int nnis_route_top(const float* logits, const float* correction, int rows, int n, int experts, int top, float* gates,
                               float* keep, void* stream) {
   NNIS_REQUIRE(logits && gates && keep, "route_top: missing operand");
@@ -389,6 +516,12 @@ extern "C" int nnis_routed_act(const void* z, int z_dtype, const float* gates, v
   NNIS_REQUIRE(nnis_dtype_ok(z_dtype) && nnis_dtype_ok(out_dtype), "routed_act: unknown dtype");
   if (rows <= 0) return 0;
   const size_t total = (size_t)rows * experts * ff;
+  if (z_dtype == NNIS_BF16 && out_dtype == NNIS_BF16 && ff % 8 == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    hipLaunchKernelGGL(routed_act_bf16x8_kernel, dim3(blocks_for(total / 8, 256)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)z, gates,
+                       (bf16_t*)out, experts, ff / 8, total / 8);
+    NNIS_LAUNCH_CHECK("routed_act");
+    return 0;
+  }
   hipLaunchKernelGGL(routed_act_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, (hipStream_t)stream, z, z_dtype, gates, out, out_dtype,
                      experts, ff, total);
   NNIS_LAUNCH_CHECK("routed_act");
@@ -453,12 +586,14 @@ extern "C" int nnis_pool_blocks(const void* k_pages, const void* v_pages, int ca
   NNIS_REQUIRE(k_pages && v_pages && block_table && pool_k && pool_v && pool_table && tok_slot && tok_pos, "pool_blocks: missing operand");
   NNIS_REQUIRE(nnis_dtype_ok(cache_dtype) && max_pages > 0 && pool_max_pages > 0, "pool_blocks: bad pages");
   NNIS_REQUIRE(kv_heads > 0 && head_dim > 0 && value_dim > 0 && pool > 0, "pool_blocks: bad sizes");
+  NNIS_REQUIRE(head_dim + value_dim <= kPoolMostChannels, "pool_blocks: a head's keys and values take up to %d channels together, got %d",
+               kPoolMostChannels, head_dim + value_dim);
   if (tokens <= 0) return 0;
   PoolArgs a;
   a.k_pages = k_pages; a.v_pages = v_pages; a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
   a.pool_k = pool_k; a.pool_v = pool_v; a.pool_table = pool_table; a.pool_max_pages = pool_max_pages;
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.kv_heads = kv_heads; a.head_dim = head_dim; a.value_dim = value_dim; a.pool = pool;
-  hipLaunchKernelGGL(pool_blocks_kernel, dim3(tokens, kv_heads), dim3(128), 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(pool_blocks_kernel, dim3(tokens, kv_heads), dim3(256), 0, (hipStream_t)stream, a);
   NNIS_LAUNCH_CHECK("pool_blocks");
   return 0;
 }

@@ -106,6 +106,7 @@ _SUBLAYER_SIGNATURES = {
     "nnis_cast_rows": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _VOID],
     "nnis_rms_post_step": [_VOID, _VOID, _INT, _VOID, _INT, _FLT, _FLT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_poly_norm": [_VOID, _INT, _VOID, _FLT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_router_logits": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_route_top": [_VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID],
     "nnis_routed_act": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_rows_axpy": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _VOID],
@@ -1886,6 +1887,20 @@ def poly_norm(z: torch.Tensor, coefficients: torch.Tensor, eps: float, out: torc
 
 
 ROUTE_MOST_OUTPUTS = 1024
+ROUTE_MOST_CHANNELS = 16384
+
+
+def router_logits(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[row, e] = x[row] . weight[e] in 32-bit: ``weight`` float32 [outputs, width], ``out`` float32 [rows, outputs];
+    ``x`` in either type."""
+    _dev(x, "x"), _dev(weight, "router weight"), _dev(out, "out")
+    rows, width = x.shape
+    if (x.dim() != 2 or not x.is_contiguous() or weight.dtype != torch.float32 or weight.dim() != 2 or weight.shape[1] != width
+            or out.dtype != torch.float32 or tuple(out.shape) != (rows, weight.shape[0]) or width > ROUTE_MOST_CHANNELS):
+        raise KernelError(f"router_logits: x {tuple(x.shape)}, a float32 weight {tuple(weight.shape)}, float32 out {tuple(out.shape)}")
+    lib = sublayer()
+    _check(lib, lib.nnis_router_logits(x.data_ptr(), _code(x), weight.data_ptr(), out.data_ptr(), rows, weight.shape[0], width, _stream()))
+    return out
 
 
 def route_top(logits: torch.Tensor, correction: Optional[torch.Tensor], experts: int, top: int, gates: torch.Tensor,

@@ -129,8 +129,9 @@ class RoutedFeedForward(FeedForward):
         return out
 
     def check(self, rt):
-        if self.experts + self.identity > rt.ops.ROUTE_MOST_OUTPUTS:
-            raise Unsupported(f"the router kernel takes up to {rt.ops.ROUTE_MOST_OUTPUTS} outputs, got {self.experts + self.identity}")
+        if self.experts + self.identity > rt.ops.ROUTE_MOST_OUTPUTS or self.width > rt.ops.ROUTE_MOST_CHANNELS:
+            raise Unsupported(f"the router kernels take up to {rt.ops.ROUTE_MOST_OUTPUTS} outputs of rows of up to "
+                              f"{rt.ops.ROUTE_MOST_CHANNELS} channels, got {self.experts + self.identity} and {self.width}")
 
     def bind(self, weights, rt):
         n = self.names
@@ -144,7 +145,7 @@ class RoutedFeedForward(FeedForward):
 
     def forward(self, x, ctx, rt):
         tokens = x.shape[0]
-        logits = rt.ops.gemm_ordered(x, self.router, rt.empty(tokens, self.experts + self.identity, dtype=torch.float32))
+        logits = rt.ops.router_logits(x, self.router, rt.empty(tokens, self.experts + self.identity, dtype=torch.float32))
         gates, keep = rt.ops.route_top(logits, self.correction, self.experts, self.top,
                                        rt.empty(tokens, self.experts, dtype=torch.float32), rt.empty(tokens, dtype=torch.float32))
         z = self.up(x, rt)

@@ -112,6 +112,18 @@ def test_poly_norm(dtype, rows, inner):
     assert _relative(got.float().cpu(), want) < (1e-6 if dtype == torch.float32 else 4e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows, outputs, width", [(1, 3, 8), (70, 11, 96), (300, 9, 200), (300, 5, 3500), (260, 70, 6500)])
+def test_router_logits_are_32_bit_products(dtype, rows, outputs, width):
+    from nnis_amd.kernels import ops
+
+    generator = torch.Generator().manual_seed(rows + width)
+    x = torch.randn(rows, width, generator=generator).to(dtype)
+    w = torch.randn(outputs, width, generator=generator)
+    got = ops.router_logits(x.cuda(), w.cuda(), torch.empty(rows, outputs, device="cuda"))
+    assert _relative(got.cpu(), x.double() @ w.double().T) < 2e-6
+
+
 @pytest.mark.parametrize("experts, identity, top", [(5, 1, 2), (3, 0, 1), (9, 2, 3), (70, 3, 4), (1, 0, 1), (2, 2, 4)])
 def test_the_router_chooses_by_corrected_scores_and_weighs_by_plain_ones(experts, identity, top):
     """The correction is large against the scores' differences, so it decides who is chosen; the weights are the

@@ -790,6 +790,7 @@ __global__ __launch_bounds__(256) void min_gru_kernel(MinGruArgs a) {
       s = fmaf(a.decay[at], s, a.ends[at]);
     }
   }
+#pragma unroll 4
   for (int t = first; t < last; ++t) {
     const size_t at = (size_t)t * a.stride + c;
     const float z = sigmoid_f(load_as_f32(a.rows, a.dtype, at) + bz);

@@ -2,7 +2,7 @@
 // route their tokens: row-wise kernels, all 32-bit inside whatever the storage type.
 //
 //   cast_rows          rows of one type as rows of another (the 32-bit stream as a sublayer's input)
-//   rms_post_step      x += y / rms(y) * (offset + w), and the stream's rows in the activation type
+//   rms_post_step      x += y / rms(y) * (offset + w), and the stream's rows in the activation type; y may stand for y + share * rows
 //   poly_norm          a N(z) + b N(z^2) + c N(z^3) + e, N a division by the root mean square of a row
 //   router_logits      a router's logits as 32-bit dot products
 //   route_top          softmax of router logits, the `top` largest of score + correction, dense weights out
@@ -31,11 +31,14 @@ constexpr int kPostKeep = 16;  // values of a row that a thread keeps in registe
 
 __global__ __launch_bounds__(256) void rms_post_step_kernel(float* __restrict__ x, const void* __restrict__ y, int y_dtype,
                                                             const void* __restrict__ weight, int w_dtype, float offset, float eps,
-                                                            void* __restrict__ h, int h_dtype, int width) {
+                                                            void* h, int h_dtype, int width, const float* __restrict__ keep,
+                                                            const void* h_in, int h_in_dtype) {
   __shared__ float scratch[16];
   const size_t base = (size_t)blockIdx.x * width;
   // everything the row needs is asked for before the sum is waited for: y, the stream and the weight, up to
   // kPostKeep values a thread; what lies beyond (rows wider than kPostKeep x the block) is read a second time
+  // with `keep`: y stands for y + keep[row] * h_in[row] (h_in may be h itself: a row is read before it is written)
+  const float share = keep ? keep[blockIdx.x] : 0.0f;
   float ys[kPostKeep], xs[kPostKeep], ws[kPostKeep];
   float ss = 0.0f;
 #pragma unroll
@@ -43,13 +46,15 @@ __global__ __launch_bounds__(256) void rms_post_step_kernel(float* __restrict__ 
     const int c = threadIdx.x + i * blockDim.x;
     if (c < width) {
       ys[i] = load_as_f32(y, y_dtype, base + c);
+      if (keep) ys[i] = fmaf(share, load_as_f32(h_in, h_in_dtype, base + c), ys[i]);
       xs[i] = x[base + c];
       ws[i] = offset + load_as_f32(weight, w_dtype, c);
       ss = fmaf(ys[i], ys[i], ss);
     }
   }
   for (int c = threadIdx.x + kPostKeep * blockDim.x; c < width; c += blockDim.x) {
-    const float v = load_as_f32(y, y_dtype, base + c);
+    float v = load_as_f32(y, y_dtype, base + c);
+    if (keep) v = fmaf(share, load_as_f32(h_in, h_in_dtype, base + c), v);
     ss = fmaf(v, v, ss);
   }
   const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
@@ -63,7 +68,8 @@ __global__ __launch_bounds__(256) void rms_post_step_kernel(float* __restrict__ 
     }
   }
   for (int c = threadIdx.x + kPostKeep * blockDim.x; c < width; c += blockDim.x) {
-    const float v = load_as_f32(y, y_dtype, base + c);
+    float v = load_as_f32(y, y_dtype, base + c);
+    if (keep) v = fmaf(share, load_as_f32(h_in, h_in_dtype, base + c), v);
     const float sum = x[base + c] + v * inv * (offset + load_as_f32(weight, w_dtype, c));
     x[base + c] = sum;
     if (h) store_from_f32(h, h_dtype, base + c, sum);
@@ -114,58 +120,24 @@ __global__ __launch_bounds__(256) void poly_norm_kernel(const void* __restrict__
 }
 
 // -----------------------------------------------------------------------------
-// A router's logits: logits[row, e] = sum_c x[row, c] * w[e, c] in 32-bit, w float32 [n, width].  A block takes R rows,
-// kept in LDS as floats; a wave takes an output at a time for all of them (lanes stride over the channels), so a row
-// of the weight is read once a block.
-// -----------------------------------------------------------------------------
-template <int R>
-__global__ __launch_bounds__(256) void router_logits_kernel(const void* __restrict__ x, int x_dtype, const float* __restrict__ w,
-                                                            float* __restrict__ logits, int rows, int n, int width) {
-  extern __shared__ float xs[];  // [R][width]
-  const int row0 = blockIdx.x * R;
-  for (int i = threadIdx.x; i < R * width; i += blockDim.x) {
-    const int r = i / width;
-    xs[i] = row0 + r < rows ? load_as_f32(x, x_dtype, (size_t)(row0 + r) * width + i % width) : 0.0f;
-  }
-  __syncthreads();
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, waves = blockDim.x / kWave;
-  for (int e = wave; e < n; e += waves) {
-    float acc[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
-    const float* row = w + (size_t)e * width;
-    for (int c = lane; c < width; c += kWave) {
-      const float wv = row[c];
-#pragma unroll
-      for (int r = 0; r < R; ++r) acc[r] = fmaf(xs[r * width + c], wv, acc[r]);
-    }
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const float total = wave_sum(acc[r]);
-      if (lane == 0 && row0 + r < rows) logits[(size_t)(row0 + r) * n + e] = total;
-    }
-  }
-}
-
-// -----------------------------------------------------------------------------
+// A router's logits are logits[row, e] = sum_c x[row, c] * w[e, c] in 32-bit, w float32 [n, width]: a block takes R
+// rows, kept in LDS as floats; a wave takes an output at a time for all of them (lanes stride over the channels), so
+// a row of the weight is read once a block.
 // Routing: scores s = softmax(logits) over n outputs; the `top` outputs with the largest s + correction are chosen
 // (the lower index on a tie); gates[row, e] = s_e for a chosen output below `experts`, 0 for the others; keep[row] =
 // the sum of s over the chosen outputs from `experts` on (those hand the input through).  A wave a row.
 // -----------------------------------------------------------------------------
 constexpr int kRouteMost = 16;  // outputs a lane holds: n <= 64 * kRouteMost
 
-__global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int rows,
-                                                        int n, int experts, int top, float* __restrict__ gates,
-                                                        float* __restrict__ keep) {
-  const int row = blockIdx.x * 4 + threadIdx.x / kWave;
-  const int lane = threadIdx.x % kWave;
-  if (row >= rows) return;
+// one row by one wave; `logits`: the row's n logits (global memory or LDS)
+__device__ __forceinline__ void route_row(const float* logits, const float* __restrict__ correction, int row, int n, int experts, int top,
+                                          float* __restrict__ gates, float* __restrict__ keep, int lane) {
   float s[kRouteMost], choice[kRouteMost];
   float top_logit = -INFINITY;
 #pragma unroll
   for (int i = 0; i < kRouteMost; ++i) {
     const int e = i * kWave + lane;
-    s[i] = e < n ? logits[(size_t)row * n + e] : -INFINITY;
+    s[i] = e < n ? logits[e] : -INFINITY;
     top_logit = fmaxf(top_logit, s[i]);
   }
   top_logit = wave_max(top_logit);
@@ -220,6 +192,102 @@ __global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict_
   }
   kept = wave_sum(kept);
   if (lane == 0) keep[row] = kept;
+}
+
+__global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int rows,
+                                                        int n, int experts, int top, float* __restrict__ gates,
+                                                        float* __restrict__ keep) {
+  const int row = blockIdx.x * 4 + threadIdx.x / kWave;
+  if (row >= rows) return;
+  route_row(logits + (size_t)row * n, correction, row, n, experts, top, gates, keep, threadIdx.x % kWave);
+}
+
+// the dot products of R rows with every output's weights, into `out` [R][n] (LDS or global memory with a row stride
+// of n); `xs`: the rows as floats in LDS [R][width].  A wave an output at a time, four channels a lane and load.
+template <int R>
+__device__ __forceinline__ void router_dots(const float* xs, const float* __restrict__ w, float* out, int n, int width) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, waves = blockDim.x / kWave;
+  for (int e = wave; e < n; e += waves) {
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+    const float* row = w + (size_t)e * width;
+    if (width % 4 == 0) {
+#pragma unroll 4
+      for (int c = 4 * lane; c < width; c += 4 * kWave) {
+        const float4 wv = *(const float4*)(row + c);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const float4 xv = *(const float4*)(xs + r * width + c);
+          acc[r] = fmaf(xv.x, wv.x, fmaf(xv.y, wv.y, fmaf(xv.z, wv.z, fmaf(xv.w, wv.w, acc[r]))));
+        }
+      }
+    } else {
+#pragma unroll 4
+      for (int c = lane; c < width; c += kWave) {
+        const float wv = row[c];
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r] = fmaf(xs[r * width + c], wv, acc[r]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float total = wave_sum(acc[r]);
+      if (lane == 0) out[r * n + e] = total;
+    }
+  }
+}
+
+// Logits and choice in one kernel: a block takes R rows (as floats in LDS), its waves the outputs' dot products into
+// LDS, then wave r routes row r.
+template <int R>
+__global__ __launch_bounds__(256) void route_kernel(const void* __restrict__ x, int x_dtype, const float* __restrict__ w,
+                                                    const float* __restrict__ correction, int rows, int n, int width, int experts,
+                                                    int top, float* __restrict__ gates, float* __restrict__ keep) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];  // [R][width] rows, then [R][n] logits
+  float* xs = lds;
+  float* lg = lds + (size_t)R * width;
+  const int row0 = blockIdx.x * R;
+  for (int i = threadIdx.x; i < R * width; i += blockDim.x) {
+    const int r = i / width;
+    xs[i] = row0 + r < rows ? load_as_f32(x, x_dtype, (size_t)(row0 + r) * width + i % width) : 0.0f;
+  }
+  __syncthreads();
+  router_dots<R>(xs, w, lg, n, width);
+  __syncthreads();
+  const int wave = threadIdx.x / kWave;
+  if (wave < R && row0 + wave < rows) route_row(lg + wave * n, correction, row0 + wave, n, experts, top, gates, keep, threadIdx.x % kWave);
+}
+
+// the logits alone, to global memory [rows, n]
+template <int R>
+__global__ __launch_bounds__(256) void router_logits_kernel(const void* __restrict__ x, int x_dtype, const float* __restrict__ w,
+                                                            float* __restrict__ logits, int rows, int n, int width) {
+  extern __shared__ __attribute__((aligned(16))) float xs[];  // [R][width]
+  const int row0 = blockIdx.x * R;
+  for (int i = threadIdx.x; i < R * width; i += blockDim.x) {
+    const int r = i / width;
+    xs[i] = row0 + r < rows ? load_as_f32(x, x_dtype, (size_t)(row0 + r) * width + i % width) : 0.0f;
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, waves = blockDim.x / kWave;
+  for (int e = wave; e < n; e += waves) {
+    const float* row = w + (size_t)e * width;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+#pragma unroll 4
+    for (int c = lane; c < width; c += kWave) {
+      const float wv = row[c];
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] = fmaf(xs[r * width + c], wv, acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float total = wave_sum(acc[r]);
+      if (lane == 0 && row0 + r < rows) logits[(size_t)(row0 + r) * n + e] = total;
+    }
+  }
 }
 
 // out[row, e * ff + c] = gates[row, e] * relu(z[row, e * ff + c])^2
@@ -386,10 +454,12 @@ struct PoolArgs {
   int kv_heads, head_dim, value_dim, pool;
 };
 
-constexpr int kPoolMostChannels = 2048;  // key and value channels of a head together
-
+// A block a (token that completes a block, key/value head).  Keys: a lane takes a token of the block, a wave a chunk of
+// eight channels at a time (sixteen or thirty-two bytes of one token, next to each other in the page); the lanes'
+// sums meet by shuffles.  Values: a page keeps eight tokens of a channel together, so a lane takes a channel and a
+// wave runs over the block's tokens.
+template <typename CacheT>
 __global__ __launch_bounds__(256) void pool_blocks_kernel(PoolArgs a) {
-  __shared__ float part[4][kPoolMostChannels];
   const int token = blockIdx.x;
   const int kv_head = blockIdx.y;
   const int slot = a.tok_slot[token];
@@ -403,31 +473,36 @@ __global__ __launch_bounds__(256) void pool_blocks_kernel(PoolArgs a) {
   const int out_at = b % kPageTokens;
   const float share = 1.0f / (float)a.pool;
   const int hd = a.head_dim, vd = a.value_dim;
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  // the block's tokens are dealt to the four waves; a wave's lanes take the channels
-  for (int d = lane; d < hd + vd; d += kWave) {
-    const bool key = d < hd;
-    const int c = key ? d : d - hd;
-    float sum = 0.0f;
-    for (int j = wave; j < a.pool; j += 4) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, waves = blockDim.x / kWave;
+  const CacheT* k_pages = (const CacheT*)a.k_pages;
+  const CacheT* v_pages = (const CacheT*)a.v_pages;
+  const size_t out = (size_t)out_page * a.kv_heads + kv_head;
+  const int chunks = (hd + 7) / 8;
+  for (int chunk = wave; chunk < chunks; chunk += waves) {
+    float sum[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j = lane; j < a.pool; j += kWave) {
       const int p = first + j;
-      const size_t page = (size_t)pages[p / kPageTokens] * a.kv_heads + kv_head;
-      sum += key ? load_as_f32(a.k_pages, a.cache_dtype, page * nnis_k_page_elems(hd) + nnis_k_offset(p % kPageTokens, c))
-                 : load_as_f32(a.v_pages, a.cache_dtype, page * nnis_v_page_elems(vd) + nnis_v_offset(c, p % kPageTokens));
+      const CacheT* at = k_pages + ((size_t)pages[p / kPageTokens] * a.kv_heads + kv_head) * nnis_k_page_elems(hd) + nnis_k_offset(p % kPageTokens, 8 * chunk);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum[e] += to_f32(at[e]);
     }
-    part[wave][d] = sum;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum[e] = wave_sum(sum[e]);
+    if (lane < 8 && 8 * chunk + lane < hd) {
+      float mine = sum[0];
+#pragma unroll
+      for (int e = 1; e < 8; ++e) mine = lane == e ? sum[e] : mine;
+      ((CacheT*)a.pool_k)[out * nnis_k_page_elems(hd) + nnis_k_offset(out_at, 8 * chunk + lane)] = from_f32<CacheT>(mine * share);
+    }
   }
-  __syncthreads();
-  for (int d = threadIdx.x; d < hd + vd; d += blockDim.x) {
-    const bool key = d < hd;
-    const int c = key ? d : d - hd;
-    const float sum = (part[0][d] + part[1][d]) + (part[2][d] + part[3][d]);
-    const size_t out = (size_t)out_page * a.kv_heads + kv_head;
-    if (key) {
-      store_from_f32(a.pool_k, a.cache_dtype, out * nnis_k_page_elems(hd) + nnis_k_offset(out_at, c), sum * share);
-    } else {
-      store_from_f32(a.pool_v, a.cache_dtype, out * nnis_v_page_elems(vd) + nnis_v_offset(c, out_at), sum * share);
+  for (int c = threadIdx.x; c < vd; c += blockDim.x) {
+    float sum = 0.0f;
+#pragma unroll 4
+    for (int j = 0; j < a.pool; ++j) {
+      const int p = first + j;
+      sum += to_f32(v_pages[((size_t)pages[p / kPageTokens] * a.kv_heads + kv_head) * nnis_v_page_elems(vd) + nnis_v_offset(c, p % kPageTokens)]);
     }
+    ((CacheT*)a.pool_v)[out * nnis_v_page_elems(vd) + nnis_v_offset(c, out_at)] = from_f32<CacheT>(sum * share);
   }
 }
 
@@ -457,12 +532,14 @@ extern "C" int nnis_cast_rows(const void* x, int x_dtype, void* out, int out_dty
 }
 
 extern "C" int nnis_rms_post_step(float* x, const void* y, int y_dtype, const void* weight, int w_dtype, float offset, float eps,
-                                  void* h, int h_dtype, int rows, int width, void* stream) {
+                                  void* h, int h_dtype, int rows, int width, const float* keep, const void* h_in, int h_in_dtype,
+                                  void* stream) {
   NNIS_REQUIRE(x && y && weight && width > 0, "rms_post_step: missing operand");
+  NNIS_REQUIRE((keep == nullptr) == (h_in == nullptr) && (h_in == nullptr || nnis_dtype_ok(h_in_dtype)), "rms_post_step: a share of rows needs both");
   NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(w_dtype) && (h == nullptr || nnis_dtype_ok(h_dtype)), "rms_post_step: unknown dtype");
   if (rows <= 0) return 0;
   hipLaunchKernelGGL(rms_post_step_kernel, dim3(rows), dim3(width >= 1024 ? 256 : (width >= 256 ? 128 : 64)), 0, (hipStream_t)stream, x, y,
-                     y_dtype, weight, w_dtype, offset, eps, h, h_dtype, width);
+                     y_dtype, weight, w_dtype, offset, eps, h, h_dtype, width, keep, h_in, h_in_dtype);
   NNIS_LAUNCH_CHECK("rms_post_step");
   return 0;
 }
@@ -495,6 +572,30 @@ extern "C" int nnis_router_logits(const void* x, int x_dtype, const float* w, fl
     hipLaunchKernelGGL((router_logits_kernel<1>), grid, dim3(256), lds, (hipStream_t)stream, x, x_dtype, w, logits, rows, n, width);
   }
   NNIS_LAUNCH_CHECK("router_logits");
+  return 0;
+}
+
+extern "C" int nnis_route(const void* x, int x_dtype, const float* w, const float* correction, int rows, int n, int width, int experts, int top,
+                          float* gates, float* keep, void* stream) {
+  NNIS_REQUIRE(x && w && gates && keep && n > 0 && width > 0, "route: missing operand");
+  NNIS_REQUIRE(nnis_dtype_ok(x_dtype), "route: unknown dtype");
+  NNIS_REQUIRE(n <= kWave * kRouteMost && width <= 8192, "route: up to %d outputs of rows of up to 8192 channels, got %d and %d", kWave * kRouteMost,
+               n, width);
+  NNIS_REQUIRE(experts >= 0 && experts <= n && top > 0 && top <= n, "route: %d experts and the %d largest of %d outputs", experts, top, n);
+  if (rows <= 0) return 0;
+  // several rows a block where they fit 48 KB of LDS and there are rows enough to fill the chip with such blocks
+  const int together = rows <= 256 ? 1 : ((size_t)4 * (width + n) * 4 <= 49152 ? 4 : ((size_t)2 * (width + n) * 4 <= 49152 ? 2 : 1));
+  const size_t lds = (size_t)together * (width + n) * sizeof(float);
+  const dim3 grid((rows + together - 1) / together);
+  hipStream_t s = (hipStream_t)stream;
+  if (together == 4) {
+    hipLaunchKernelGGL((route_kernel<4>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep);
+  } else if (together == 2) {
+    hipLaunchKernelGGL((route_kernel<2>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep);
+  } else {
+    hipLaunchKernelGGL((route_kernel<1>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep);
+  }
+  NNIS_LAUNCH_CHECK("route");
   return 0;
 }
 
@@ -586,14 +687,16 @@ extern "C" int nnis_pool_blocks(const void* k_pages, const void* v_pages, int ca
   NNIS_REQUIRE(k_pages && v_pages && block_table && pool_k && pool_v && pool_table && tok_slot && tok_pos, "pool_blocks: missing operand");
   NNIS_REQUIRE(nnis_dtype_ok(cache_dtype) && max_pages > 0 && pool_max_pages > 0, "pool_blocks: bad pages");
   NNIS_REQUIRE(kv_heads > 0 && head_dim > 0 && value_dim > 0 && pool > 0, "pool_blocks: bad sizes");
-  NNIS_REQUIRE(head_dim + value_dim <= kPoolMostChannels, "pool_blocks: a head's keys and values take up to %d channels together, got %d",
-               kPoolMostChannels, head_dim + value_dim);
   if (tokens <= 0) return 0;
   PoolArgs a;
   a.k_pages = k_pages; a.v_pages = v_pages; a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
   a.pool_k = pool_k; a.pool_v = pool_v; a.pool_table = pool_table; a.pool_max_pages = pool_max_pages;
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.kv_heads = kv_heads; a.head_dim = head_dim; a.value_dim = value_dim; a.pool = pool;
-  hipLaunchKernelGGL(pool_blocks_kernel, dim3(tokens, kv_heads), dim3(256), 0, (hipStream_t)stream, a);
+  if (cache_dtype == NNIS_F32) {
+    hipLaunchKernelGGL(pool_blocks_kernel<float>, dim3(tokens, kv_heads), dim3(256), 0, (hipStream_t)stream, a);
+  } else {
+    hipLaunchKernelGGL(pool_blocks_kernel<bf16_t>, dim3(tokens, kv_heads), dim3(256), 0, (hipStream_t)stream, a);
+  }
   NNIS_LAUNCH_CHECK("pool_blocks");
   return 0;
 }

@@ -104,7 +104,8 @@ _RECURRENT_SIGNATURES = {
 
 _SUBLAYER_SIGNATURES = {
     "nnis_cast_rows": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _VOID],
-    "nnis_rms_post_step": [_VOID, _VOID, _INT, _VOID, _INT, _FLT, _FLT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_rms_post_step": [_VOID, _VOID, _INT, _VOID, _INT, _FLT, _FLT, _VOID, _INT, _INT, _INT, _VOID, _VOID, _INT, _VOID],
+    "nnis_route": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID],
     "nnis_poly_norm": [_VOID, _INT, _VOID, _FLT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_router_logits": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_route_top": [_VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID],
@@ -1858,9 +1859,10 @@ def cast_rows(x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] =
 
 
 def rms_post_step(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, offset: float, eps: float,
-                  h: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                  h: Optional[torch.Tensor] = None, share=None) -> Optional[torch.Tensor]:
     """x += y / sqrt(mean(y^2) + eps) * (offset + weight), row by row, in place in the 32-bit stream ``x``; ``h`` (of
-    x's shape, any type) receives the new rows."""
+    x's shape, any type) receives the new rows.  ``share``: (keep float32 [rows], rows of x's shape): y then stands
+    for y + keep[row] * rows[row]; the rows may be ``h`` or ``x`` themselves."""
     _dev(x, "x"), _dev(y, "y"), _dev(weight, "norm weight")
     if x.dtype != torch.float32 or x.dim() != 2 or y.shape != x.shape or weight.numel() != x.shape[1]:
         raise KernelError(f"rms_post_step: a float32 stream {tuple(x.shape)} against y {tuple(y.shape)} and a weight of {weight.numel()}")
@@ -1869,8 +1871,15 @@ def rms_post_step(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, offset
         if h.shape != x.shape:
             raise KernelError(f"rms_post_step: h {tuple(h.shape)} against the stream {tuple(x.shape)}")
     lib = sublayer()
+    keep = rows_in = None
+    if share is not None:
+        keep, rows_in = share
+        _dev(keep, "keep"), _dev(rows_in, "shared rows")
+        if keep.dtype != torch.float32 or keep.numel() != x.shape[0] or rows_in.shape != x.shape or not rows_in.is_contiguous():
+            raise KernelError(f"rms_post_step: a float32 share per row and rows {tuple(x.shape)}, got {tuple(keep.shape)} and {tuple(rows_in.shape)}")
     _check(lib, lib.nnis_rms_post_step(x.data_ptr(), y.data_ptr(), _code(y), weight.data_ptr(), _code(weight), float(offset), float(eps),
-                                       _ptr(h), _code(h) if h is not None else 0, x.shape[0], x.shape[1], _stream()))
+                                       _ptr(h), _code(h) if h is not None else 0, x.shape[0], x.shape[1], _ptr(keep), _ptr(rows_in),
+                                       _code(rows_in) if rows_in is not None else 0, _stream()))
     return h
 
 
@@ -1921,6 +1930,30 @@ def route_top(logits: torch.Tensor, correction: Optional[torch.Tensor], experts:
         raise KernelError(f"route_top: {experts} experts and the {top} largest of {n} outputs (at most {ROUTE_MOST_OUTPUTS})")
     lib = sublayer()
     _check(lib, lib.nnis_route_top(logits.data_ptr(), _ptr(correction), rows, n, experts, top, gates.data_ptr(), keep.data_ptr(), _stream()))
+    return gates, keep
+
+
+ROUTE_FUSED_MOST_CHANNELS = 8192
+
+
+def route(x: torch.Tensor, weight: torch.Tensor, correction: Optional[torch.Tensor], experts: int, top: int, gates: torch.Tensor,
+          keep: torch.Tensor):
+    """``router_logits`` and ``route_top`` in one kernel (rows of up to ``ROUTE_FUSED_MOST_CHANNELS`` channels)."""
+    _dev(x, "x"), _dev(weight, "router weight"), _dev(gates, "gates"), _dev(keep, "keep")
+    rows, width = x.shape
+    n = weight.shape[0]
+    if (x.dim() != 2 or not x.is_contiguous() or weight.dtype != torch.float32 or weight.dim() != 2 or weight.shape[1] != width
+            or gates.dtype != torch.float32 or keep.dtype != torch.float32 or tuple(gates.shape) != (rows, experts) or keep.numel() != rows):
+        raise KernelError(f"route: x {tuple(x.shape)}, a float32 weight {tuple(weight.shape)}, float32 gates {tuple(gates.shape)} and keep {tuple(keep.shape)}")
+    if correction is not None:
+        _dev(correction, "correction")
+        if correction.dtype != torch.float32 or correction.numel() != n:
+            raise KernelError(f"route: a float32 correction per output ({n}), got {tuple(correction.shape)} {correction.dtype}")
+    if not (0 < n <= ROUTE_MOST_OUTPUTS and 0 <= experts <= n and 0 < top <= n and width <= ROUTE_FUSED_MOST_CHANNELS):
+        raise KernelError(f"route: {experts} experts and the {top} largest of {n} outputs (at most {ROUTE_MOST_OUTPUTS}) of rows of {width} channels")
+    lib = sublayer()
+    _check(lib, lib.nnis_route(x.data_ptr(), _code(x), weight.data_ptr(), _ptr(correction), rows, n, width, experts, top, gates.data_ptr(),
+                               keep.data_ptr(), _stream()))
     return gates, keep
 
 

@@ -372,7 +372,13 @@ class PostNormBlock(Block):
             h = self.entry.forward(x, rt)
         h = self.norm1.post_step(x, self.mixer.forward(h, ctx, view, rt), rt)
         if self.feed_forward is not None:
-            h = self.norm2.post_step(x, self.feed_forward.forward(h, ctx, rt), rt)
+            if getattr(self.feed_forward, "can_leave_share", False):
+                # (a feed-forward that hands a share of its input through leaves that sum to the way out's kernel)
+                y = self.feed_forward.forward(h, ctx, rt, share_later=True)
+                y, share = y if isinstance(y, tuple) else (y, None)
+                h = self.norm2.post_step(x, y, rt, share=share)
+            else:
+                h = self.norm2.post_step(x, self.feed_forward.forward(h, ctx, rt), rt)
         if following is not None and type(following) is type(self.entry):
             return PreparedRows(following, x, h)
         return x, None

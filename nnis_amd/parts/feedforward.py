@@ -143,13 +143,21 @@ class RoutedFeedForward(FeedForward):
     def weight_bytes(self):
         return self.up.weight_bytes() + self.down.weight_bytes() + self.router.numel() * 4
 
-    def forward(self, x, ctx, rt):
+    can_leave_share = True  # ``forward(..., share_later=True)`` leaves the identity outputs' share to a consumer that adds it in a kernel of its own
+
+    def forward(self, x, ctx, rt, share_later=False):
+        """With ``share_later`` and identity outputs: returns (y, (keep, x)), where the output is y + keep[row] * x[row]."""
         tokens = x.shape[0]
-        logits = rt.ops.router_logits(x, self.router, rt.empty(tokens, self.experts + self.identity, dtype=torch.float32))
-        gates, keep = rt.ops.route_top(logits, self.correction, self.experts, self.top,
-                                       rt.empty(tokens, self.experts, dtype=torch.float32), rt.empty(tokens, dtype=torch.float32))
+        gates, keep = rt.empty(tokens, self.experts, dtype=torch.float32), rt.empty(tokens, dtype=torch.float32)
+        if self.width <= rt.ops.ROUTE_FUSED_MOST_CHANNELS:
+            rt.ops.route(x, self.router, self.correction, self.experts, self.top, gates, keep)
+        else:
+            logits = rt.ops.router_logits(x, self.router, rt.empty(tokens, self.experts + self.identity, dtype=torch.float32))
+            rt.ops.route_top(logits, self.correction, self.experts, self.top, gates, keep)
         z = self.up(x, rt)
         y = self.down(rt.ops.routed_act(z, gates, rt.empty(tokens, self.experts * self.inner)), rt)
+        if self.identity and share_later:
+            return y, (keep, x)
         if self.identity:
             rt.ops.rows_axpy(y, x, keep)
         return y

@@ -46,13 +46,14 @@ class RMSNorm(Norm):
     def add_forward(self, residual, delta, rt, rows=None):
         return rt.ops.rmsnorm(residual, self.weight, self.eps, self._out(residual, rt, rows), delta=delta, rows=rows)
 
-    def post_step(self, x, y, rt):
+    def post_step(self, x, y, rt, share=None):
         """x += this norm of y, in place in the 32-bit stream; returns the new rows in the activation type (the stream
-        itself under a 32-bit runtime): what a sublayer that reads the stream un-normed takes next."""
+        itself under a 32-bit runtime): what a sublayer that reads the stream un-normed takes next.  ``share``: (a
+        factor per row, rows): y stands for y + factor * rows (a sublayer's share of its own input, left to this kernel)."""
         if rt.dtype == torch.float32:
-            rt.ops.rms_post_step(x, y, self.weight, 0.0, self.eps)
+            rt.ops.rms_post_step(x, y, self.weight, 0.0, self.eps, share=share)
             return x
-        return rt.ops.rms_post_step(x, y, self.weight, 0.0, self.eps, h=rt.empty(x.shape[0], self.width))
+        return rt.ops.rms_post_step(x, y, self.weight, 0.0, self.eps, h=rt.empty(x.shape[0], self.width), share=share)
 
 
 register_init_rule("small", lambda spec, generator, dtype: (0.1 * torch.randn(tuple(spec.shape), generator=generator)).to(dtype),

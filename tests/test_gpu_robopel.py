@@ -93,6 +93,13 @@ def test_the_norm_on_the_way_out(y_dtype, tokens, width):
     stream = x.clone().cuda()
     ops.rms_post_step(stream, y.cuda(), (1.0 + w).cuda(), 0.0, 1e-5)  # (the offset added beforehand, no rows asked for)
     assert _relative(stream.cpu(), want) < 1e-6
+    # a share of other rows joins y before the norm; the rows may be the very buffer that receives the new ones
+    keep = torch.rand(tokens, generator=generator)
+    rows_in = torch.randn(tokens, width, generator=generator).to(torch.bfloat16)
+    want = x.double() + R.rms_norm(y.double() + keep.double()[:, None] * rows_in.double(), 1.0 + w.double(), 1e-5)
+    stream, rows = x.clone().cuda(), rows_in.clone().cuda()
+    ops.rms_post_step(stream, y.cuda(), w.cuda(), 1.0, 1e-5, h=rows, share=(keep.cuda(), rows))
+    assert _relative(stream.cpu(), want) < 1e-6 and _relative(rows.float().cpu(), want) < 4e-3
     picked = torch.tensor([tokens - 1, 0], dtype=torch.int32).cuda()
     got = ops.cast_rows(stream, torch.empty(2, width, device="cuda", dtype=torch.bfloat16), picked)
     assert torch.equal(got.cpu(), stream.cpu()[[tokens - 1, 0]].to(torch.bfloat16))
@@ -122,6 +129,19 @@ def test_router_logits_are_32_bit_products(dtype, rows, outputs, width):
     w = torch.randn(outputs, width, generator=generator)
     got = ops.router_logits(x.cuda(), w.cuda(), torch.empty(rows, outputs, device="cuda"))
     assert _relative(got.cpu(), x.double() @ w.double().T) < 2e-6
+    # logits and choice in one kernel give what the two kernels give
+    experts, top = max(1, outputs - 2), min(3, outputs)
+    correction = 0.3 * torch.randn(outputs, generator=generator)
+    apart = ops.route_top(got, correction.cuda(), experts, top, torch.empty(rows, experts, device="cuda"), torch.empty(rows, device="cuda"))
+    fused = ops.route(x.cuda(), w.cuda(), correction.cuda(), experts, top, torch.empty(rows, experts, device="cuda"), torch.empty(rows, device="cuda"))
+    scores = torch.softmax((x.double() @ w.double().T), dim=-1)
+    for one, other in zip(apart, fused):
+        close = (one - other).abs() < 1e-5
+        # (a choice may differ where two corrected scores are closer than the two sums' rounding)
+        assert float(close.float().mean()) > 0.995, float(close.float().mean())
+    chosen = torch.topk(scores + correction.double(), top, dim=-1).indices
+    total = fused[0].cpu().double().sum(dim=1) + fused[1].cpu().double()  # a row's weights, identity outputs included
+    assert float(((total - scores.gather(1, chosen).sum(dim=1)).abs() < 1e-5).float().mean()) > 0.995
 
 
 @pytest.mark.parametrize("experts, identity, top", [(5, 1, 2), (3, 0, 1), (9, 2, 3), (70, 3, 4), (1, 0, 1), (2, 2, 4)])

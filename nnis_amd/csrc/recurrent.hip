@@ -785,7 +785,8 @@ __global__ __launch_bounds__(256) void min_gru_kernel(MinGruArgs a) {
   } else {
     // what the pieces before this one hand on: the first piece's end, then I <- decay_k I + ends_k piece by piece
     s = a.ends[(size_t)b * a.pieces * a.width + c];
-    for (int k = 1; k < piece; ++k) {
+#pragma unroll 8
+    for (int k = 1; k < piece; ++k) {  // (the loads do not wait for the sums: eight pieces' are asked for at a time)
       const size_t at = ((size_t)b * a.pieces + k) * a.width + c;
       s = fmaf(a.decay[at], s, a.ends[at]);
     }

@@ -458,6 +458,8 @@ struct PoolArgs {
 // eight channels at a time (sixteen or thirty-two bytes of one token, next to each other in the page); the lanes'
 // sums meet by shuffles.  Values: a page keeps eight tokens of a channel together, so a lane takes a channel and a
 // wave runs over the block's tokens.
+constexpr int kPoolMostValueChannels = 4096;  // (the waves' sums of a head's values meet in LDS)
+
 template <typename CacheT>
 __global__ __launch_bounds__(256) void pool_blocks_kernel(PoolArgs a) {
   const int token = blockIdx.x;
@@ -495,13 +497,30 @@ __global__ __launch_bounds__(256) void pool_blocks_kernel(PoolArgs a) {
       ((CacheT*)a.pool_k)[out * nnis_k_page_elems(hd) + nnis_k_offset(out_at, 8 * chunk + lane)] = from_f32<CacheT>(mine * share);
     }
   }
+  // values: lanes on channels, waves on the groups of eight tokens that a page keeps together for a channel (the
+  // block's first and last group may reach beyond it: those tokens are left out); the waves' sums meet in LDS
+  extern __shared__ float part_lds[];  // [waves][vd]
+  const int group_first = first / 8, group_last = (first + a.pool - 1) / 8;
+  for (int c0 = 0; c0 < vd; c0 += kWave) {
+    const int c = c0 + lane;
+    float sum = 0.0f;
+    if (c < vd) {
+      for (int group = group_first + wave; group <= group_last; group += waves) {
+        const int p0 = 8 * group;
+        const CacheT* at = v_pages + ((size_t)pages[p0 / kPageTokens] * a.kv_heads + kv_head) * nnis_v_page_elems(vd) + nnis_v_offset(c, p0 % kPageTokens);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float v = to_f32(at[e]);
+          sum += (p0 + e >= first && p0 + e < first + a.pool) ? v : 0.0f;
+        }
+      }
+      part_lds[wave * vd + c] = sum;
+    }
+  }
+  __syncthreads();
   for (int c = threadIdx.x; c < vd; c += blockDim.x) {
     float sum = 0.0f;
-#pragma unroll 4
-    for (int j = 0; j < a.pool; ++j) {
-      const int p = first + j;
-      sum += to_f32(v_pages[((size_t)pages[p / kPageTokens] * a.kv_heads + kv_head) * nnis_v_page_elems(vd) + nnis_v_offset(c, p % kPageTokens)]);
-    }
+    for (int w = 0; w < waves; ++w) sum += part_lds[w * vd + c];
     ((CacheT*)a.pool_v)[out * nnis_v_page_elems(vd) + nnis_v_offset(c, out_at)] = from_f32<CacheT>(sum * share);
   }
 }
@@ -687,15 +706,16 @@ extern "C" int nnis_pool_blocks(const void* k_pages, const void* v_pages, int ca
   NNIS_REQUIRE(k_pages && v_pages && block_table && pool_k && pool_v && pool_table && tok_slot && tok_pos, "pool_blocks: missing operand");
   NNIS_REQUIRE(nnis_dtype_ok(cache_dtype) && max_pages > 0 && pool_max_pages > 0, "pool_blocks: bad pages");
   NNIS_REQUIRE(kv_heads > 0 && head_dim > 0 && value_dim > 0 && pool > 0, "pool_blocks: bad sizes");
+  NNIS_REQUIRE(value_dim <= kPoolMostValueChannels, "pool_blocks: values of up to %d channels, got %d", kPoolMostValueChannels, value_dim);
   if (tokens <= 0) return 0;
   PoolArgs a;
   a.k_pages = k_pages; a.v_pages = v_pages; a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
   a.pool_k = pool_k; a.pool_v = pool_v; a.pool_table = pool_table; a.pool_max_pages = pool_max_pages;
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.kv_heads = kv_heads; a.head_dim = head_dim; a.value_dim = value_dim; a.pool = pool;
   if (cache_dtype == NNIS_F32) {
-    hipLaunchKernelGGL(pool_blocks_kernel<float>, dim3(tokens, kv_heads), dim3(256), 0, (hipStream_t)stream, a);
+    hipLaunchKernelGGL(pool_blocks_kernel<float>, dim3(tokens, kv_heads), dim3(256), (size_t)4 * value_dim * sizeof(float), (hipStream_t)stream, a);
   } else {
-    hipLaunchKernelGGL(pool_blocks_kernel<bf16_t>, dim3(tokens, kv_heads), dim3(256), 0, (hipStream_t)stream, a);
+    hipLaunchKernelGGL(pool_blocks_kernel<bf16_t>, dim3(tokens, kv_heads), dim3(256), (size_t)4 * value_dim * sizeof(float), (hipStream_t)stream, a);
   }
   NNIS_LAUNCH_CHECK("pool_blocks");
   return 0;

@@ -325,7 +325,9 @@ class GatedWindowAttention(Mixer):
         return self._pooled_request()
 
     def check(self, rt):
-        rt.ops.attention_check(self.head_dim, self.value_dim)
+        # (heads wider than the matrix-core kernels carry take the row kernel, at its pace)
+        wide = max(self.head_dim, self.value_dim) > rt.ops.ATTENTION_MOST_CHANNELS
+        rt.ops.attention_check(self.head_dim, self.value_dim, rt.ops.ATTENTION_ROWS_MOST_CHANNELS if wide else rt.ops.ATTENTION_MOST_CHANNELS)
         rot_dim = getattr(self.position, "rot_dim", 0)
         if rot_dim > self.head_dim:
             raise InvalidInput(f"a rotation of {rot_dim} channels does not fit heads of {self.head_dim}")

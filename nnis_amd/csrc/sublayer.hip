@@ -29,7 +29,7 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf
 // -----------------------------------------------------------------------------
 constexpr int kPostKeep = 16;  // values of a row that a thread keeps in registers between the two passes
 
-__global__ __launch_bounds__(256) void rms_post_step_kernel(float* __restrict__ x, const void* __restrict__ y, int y_dtype,
+__global__ __launch_bounds__(256) void rms_post_step_kernel(float* x, const void* __restrict__ y, int y_dtype,
                                                             const void* __restrict__ weight, int w_dtype, float offset, float eps,
                                                             void* h, int h_dtype, int width, const float* __restrict__ keep,
                                                             const void* h_in, int h_in_dtype) {
@@ -76,6 +76,64 @@ __global__ __launch_bounds__(256) void rms_post_step_kernel(float* __restrict__ 
   }
 }
 
+// The same, four channels a thread and access (rows of a multiple of four channels, a 32-bit weight): y and the
+// rows out in one type T (bfloat16 with rows out, or 32-bit), the shared rows in T too.
+__device__ __forceinline__ float4 load4(const float* p) { return *(const float4*)p; }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+  const bf16x4_t v = *(const bf16x4_t*)p;
+  return make_float4((float)v[0], (float)v[1], (float)v[2], (float)v[3]);
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *(float4*)p = v; }
+__device__ __forceinline__ void store4(bf16_t* p, float4 v) {
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+  bf16x4_t o;
+  o[0] = (__bf16)v.x; o[1] = (__bf16)v.y; o[2] = (__bf16)v.z; o[3] = (__bf16)v.w;
+  *(bf16x4_t*)p = o;
+}
+
+constexpr int kPostKeep4 = 4;  // groups of four channels that a thread keeps: rows of up to 16 x the block's threads
+
+template <typename T>
+__global__ __launch_bounds__(256) void rms_post_step4_kernel(float* x, const T* __restrict__ y, const float* __restrict__ weight,
+                                                             float offset, float eps, T* h, int width, const float* __restrict__ keep,
+                                                             const T* h_in) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * width;
+  const float share = keep ? keep[blockIdx.x] : 0.0f;
+  float4 ys[kPostKeep4], xs[kPostKeep4], ws[kPostKeep4];
+  float ss = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kPostKeep4; ++i) {
+    const int c = 4 * (threadIdx.x + i * blockDim.x);
+    if (c < width) {
+      ys[i] = load4(y + base + c);
+      xs[i] = load4(x + base + c);
+      ws[i] = load4(weight + c);
+      if (keep) {
+        const float4 r = load4(h_in + base + c);
+        ys[i].x = fmaf(share, r.x, ys[i].x); ys[i].y = fmaf(share, r.y, ys[i].y);
+        ys[i].z = fmaf(share, r.z, ys[i].z); ys[i].w = fmaf(share, r.w, ys[i].w);
+      }
+      ss = fmaf(ys[i].x, ys[i].x, fmaf(ys[i].y, ys[i].y, fmaf(ys[i].z, ys[i].z, fmaf(ys[i].w, ys[i].w, ss))));
+    }
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+#pragma unroll
+  for (int i = 0; i < kPostKeep4; ++i) {
+    const int c = 4 * (threadIdx.x + i * blockDim.x);
+    if (c < width) {
+      float4 sum;
+      sum.x = xs[i].x + ys[i].x * inv * (offset + ws[i].x);
+      sum.y = xs[i].y + ys[i].y * inv * (offset + ws[i].y);
+      sum.z = xs[i].z + ys[i].z * inv * (offset + ws[i].z);
+      sum.w = xs[i].w + ys[i].w * inv * (offset + ws[i].w);
+      store4(x + base + c, sum);
+      if (h) store4(h + base + c, sum);
+    }
+  }
+}
+
 // -----------------------------------------------------------------------------
 // PolyNorm: out = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e, powers element by element, each root mean
 // square over the row with eps inside the root; coef = (a, b, c, e) in device memory.
@@ -116,6 +174,43 @@ __global__ __launch_bounds__(256) void poly_norm_kernel(const void* __restrict__
   for (int c = threadIdx.x + kPolyKeep * blockDim.x; c < width; c += blockDim.x) {
     const float v = load_as_f32(z, z_dtype, base + c);
     store_from_f32(out, out_dtype, base + c, fmaf(v, fmaf(v, fmaf(v, cc, b), a), e));
+  }
+}
+
+// the same, four values a thread and access (rows of a multiple of four, in and out of one type)
+constexpr int kPolyKeep4 = 8;  // groups of four that a thread keeps: rows of up to 32 x the block's threads
+
+template <typename T>
+__global__ __launch_bounds__(256) void poly_norm4_kernel(const T* __restrict__ z, const float* __restrict__ coef, float eps, T* __restrict__ out,
+                                                         int width) {
+  __shared__ float scratch[3][16];
+  const size_t base = (size_t)blockIdx.x * width;
+  float4 zs[kPolyKeep4];
+  float s2 = 0.0f, s4 = 0.0f, s6 = 0.0f;
+  auto add = [&](float v) {
+    const float v2 = v * v;
+    s2 += v2;
+    s4 = fmaf(v2, v2, s4);
+    s6 = fmaf(v2 * v, v2 * v, s6);
+  };
+#pragma unroll
+  for (int i = 0; i < kPolyKeep4; ++i) {
+    const int c = 4 * (threadIdx.x + i * blockDim.x);
+    if (c < width) {
+      zs[i] = load4(z + base + c);
+      add(zs[i].x), add(zs[i].y), add(zs[i].z), add(zs[i].w);
+    }
+  }
+  const float n = (float)width;
+  const float i1 = 1.0f / sqrtf(block_sum(s2, scratch[0]) / n + eps);
+  const float i2 = 1.0f / sqrtf(block_sum(s4, scratch[1]) / n + eps);
+  const float i3 = 1.0f / sqrtf(block_sum(s6, scratch[2]) / n + eps);
+  const float a = coef[0] * i1, b = coef[1] * i2, cc = coef[2] * i3, e = coef[3];
+  auto act = [&](float v) { return fmaf(v, fmaf(v, fmaf(v, cc, b), a), e); };
+#pragma unroll
+  for (int i = 0; i < kPolyKeep4; ++i) {
+    const int c = 4 * (threadIdx.x + i * blockDim.x);
+    if (c < width) store4(out + base + c, make_float4(act(zs[i].x), act(zs[i].y), act(zs[i].z), act(zs[i].w)));
   }
 }
 
@@ -437,7 +532,10 @@ __global__ __launch_bounds__(64) void head_norm_write_kernel(HeadWriteArgs a) {
 // -----------------------------------------------------------------------------
 // Pooled blocks: a token at position p with (p + 1) % pool == 0 completes block b = p / pool of its sequence; the
 // block's key is the mean of its `pool` keys as the pages hold them, its value the mean of their values; both go to
-// entry b of a second set of pages with a block table of its own.  Runs behind the step's cache write.
+// entry b of a second set of pages with a block table of its own.  Runs behind the step's cache write.  A sequence
+// that brings n tokens from position p0 completes (p0 + n) / pool - p0 / pool blocks; the launch has a block for every
+// one that the step's sequences can complete between them (tokens / pool + sequences), and each finds its
+// (sequence, block) by counting through the sequences.
 // -----------------------------------------------------------------------------
 struct PoolArgs {
   const void* k_pages;
@@ -449,8 +547,10 @@ struct PoolArgs {
   void* pool_v;
   const int* pool_table;
   int pool_max_pages;
-  const int* tok_slot;
-  const int* tok_pos;
+  const int* seq_slot;
+  const int* seq_start;
+  const int* seq_pos0;
+  int batch;
   int kv_heads, head_dim, value_dim, pool;
 };
 
@@ -462,13 +562,21 @@ constexpr int kPoolMostValueChannels = 4096;  // (the waves' sums of a head's va
 
 template <typename CacheT>
 __global__ __launch_bounds__(256) void pool_blocks_kernel(PoolArgs a) {
-  const int token = blockIdx.x;
   const int kv_head = blockIdx.y;
-  const int slot = a.tok_slot[token];
-  if (slot < 0) return;
-  const int pos = a.tok_pos[token];
-  if ((pos + 1) % a.pool != 0) return;
-  const int b = pos / a.pool;
+  int left = blockIdx.x, slot = -1, b = 0;
+  for (int i = 0; i < a.batch; ++i) {
+    const int s = a.seq_slot[i];
+    if (s < 0) continue;  // a padding row
+    const int p0 = a.seq_pos0[i], n = a.seq_start[i + 1] - a.seq_start[i];
+    const int count = (p0 + n) / a.pool - p0 / a.pool;
+    if (left < count) {
+      slot = s;
+      b = p0 / a.pool + left;
+      break;
+    }
+    left -= count;
+  }
+  if (slot < 0) return;  // fewer blocks were completed than the launch has room for
   const int first = b * a.pool;
   const int* pages = a.block_table + (size_t)slot * a.max_pages;
   const int out_page = a.pool_table[(size_t)slot * a.pool_max_pages + b / kPageTokens];
@@ -557,6 +665,23 @@ extern "C" int nnis_rms_post_step(float* x, const void* y, int y_dtype, const vo
   NNIS_REQUIRE((keep == nullptr) == (h_in == nullptr) && (h_in == nullptr || nnis_dtype_ok(h_in_dtype)), "rms_post_step: a share of rows needs both");
   NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(w_dtype) && (h == nullptr || nnis_dtype_ok(h_dtype)), "rms_post_step: unknown dtype");
   if (rows <= 0) return 0;
+  // four channels a thread where the types and the row's length allow
+  const int threads4 = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
+  const bool fits4 = width % 4 == 0 && width <= 4 * kPostKeep4 * threads4 && w_dtype == NNIS_F32 && (uintptr_t)y % 16 == 0 &&
+                     (uintptr_t)weight % 16 == 0 && (h == nullptr || (uintptr_t)h % 16 == 0) && (h_in == nullptr || (uintptr_t)h_in % 16 == 0) &&
+                     (h_in == nullptr || h_in_dtype == y_dtype);
+  if (fits4 && y_dtype == NNIS_BF16 && (h == nullptr || h_dtype == NNIS_BF16)) {
+    hipLaunchKernelGGL(rms_post_step4_kernel<bf16_t>, dim3(rows), dim3(threads4), 0, (hipStream_t)stream, x, (const bf16_t*)y,
+                       (const float*)weight, offset, eps, (bf16_t*)h, width, keep, (const bf16_t*)h_in);
+    NNIS_LAUNCH_CHECK("rms_post_step");
+    return 0;
+  }
+  if (fits4 && y_dtype == NNIS_F32 && (h == nullptr || h_dtype == NNIS_F32)) {
+    hipLaunchKernelGGL(rms_post_step4_kernel<float>, dim3(rows), dim3(threads4), 0, (hipStream_t)stream, x, (const float*)y,
+                       (const float*)weight, offset, eps, (float*)h, width, keep, (const float*)h_in);
+    NNIS_LAUNCH_CHECK("rms_post_step");
+    return 0;
+  }
   hipLaunchKernelGGL(rms_post_step_kernel, dim3(rows), dim3(width >= 1024 ? 256 : (width >= 256 ? 128 : 64)), 0, (hipStream_t)stream, x, y,
                      y_dtype, weight, w_dtype, offset, eps, h, h_dtype, width, keep, h_in, h_in_dtype);
   NNIS_LAUNCH_CHECK("rms_post_step");
@@ -568,6 +693,16 @@ extern "C" int nnis_poly_norm(const void* z, int z_dtype, const float* coef, flo
   NNIS_REQUIRE(z && coef && out && width > 0, "poly_norm: missing operand");
   NNIS_REQUIRE(nnis_dtype_ok(z_dtype) && nnis_dtype_ok(out_dtype), "poly_norm: unknown dtype");
   if (rows <= 0) return 0;
+  const int threads4 = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
+  if (width % 4 == 0 && width <= 4 * kPolyKeep4 * threads4 && z_dtype == out_dtype && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    if (z_dtype == NNIS_BF16) {
+      hipLaunchKernelGGL(poly_norm4_kernel<bf16_t>, dim3(rows), dim3(threads4), 0, (hipStream_t)stream, (const bf16_t*)z, coef, eps, (bf16_t*)out, width);
+    } else {
+      hipLaunchKernelGGL(poly_norm4_kernel<float>, dim3(rows), dim3(threads4), 0, (hipStream_t)stream, (const float*)z, coef, eps, (float*)out, width);
+    }
+    NNIS_LAUNCH_CHECK("poly_norm");
+    return 0;
+  }
   hipLaunchKernelGGL(poly_norm_kernel, dim3(rows), dim3(width >= 1024 ? 256 : (width >= 256 ? 128 : 64)), 0, (hipStream_t)stream, z, z_dtype,
                      coef, eps, out, out_dtype, width);
   NNIS_LAUNCH_CHECK("poly_norm");
@@ -701,21 +836,23 @@ extern "C" int nnis_head_norm_write(const void* rows, int dtype, int stride, int
 }
 
 extern "C" int nnis_pool_blocks(const void* k_pages, const void* v_pages, int cache_dtype, const int* block_table, int max_pages,
-                                void* pool_k, void* pool_v, const int* pool_table, int pool_max_pages, const int* tok_slot,
-                                const int* tok_pos, int tokens, int kv_heads, int head_dim, int value_dim, int pool, void* stream) {
-  NNIS_REQUIRE(k_pages && v_pages && block_table && pool_k && pool_v && pool_table && tok_slot && tok_pos, "pool_blocks: missing operand");
+                                void* pool_k, void* pool_v, const int* pool_table, int pool_max_pages, const int* seq_slot,
+                                const int* seq_start, const int* seq_pos0, int batch, int tokens, int kv_heads, int head_dim,
+                                int value_dim, int pool, void* stream) {
+  NNIS_REQUIRE(k_pages && v_pages && block_table && pool_k && pool_v && pool_table && seq_slot && seq_start && seq_pos0,
+               "pool_blocks: missing operand");
   NNIS_REQUIRE(nnis_dtype_ok(cache_dtype) && max_pages > 0 && pool_max_pages > 0, "pool_blocks: bad pages");
   NNIS_REQUIRE(kv_heads > 0 && head_dim > 0 && value_dim > 0 && pool > 0, "pool_blocks: bad sizes");
   NNIS_REQUIRE(value_dim <= kPoolMostValueChannels, "pool_blocks: values of up to %d channels, got %d", kPoolMostValueChannels, value_dim);
-  if (tokens <= 0) return 0;
+  if (tokens <= 0 || batch <= 0) return 0;
   PoolArgs a;
   a.k_pages = k_pages; a.v_pages = v_pages; a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
   a.pool_k = pool_k; a.pool_v = pool_v; a.pool_table = pool_table; a.pool_max_pages = pool_max_pages;
-  a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.kv_heads = kv_heads; a.head_dim = head_dim; a.value_dim = value_dim; a.pool = pool;
+  a.seq_slot = seq_slot; a.seq_start = seq_start; a.seq_pos0 = seq_pos0; a.batch = batch; a.kv_heads = kv_heads; a.head_dim = head_dim; a.value_dim = value_dim; a.pool = pool;
   if (cache_dtype == NNIS_F32) {
-    hipLaunchKernelGGL(pool_blocks_kernel<float>, dim3(tokens, kv_heads), dim3(256), (size_t)4 * value_dim * sizeof(float), (hipStream_t)stream, a);
+    hipLaunchKernelGGL(pool_blocks_kernel<float>, dim3(tokens / pool + batch, kv_heads), dim3(256), (size_t)4 * value_dim * sizeof(float), (hipStream_t)stream, a);
   } else {
-    hipLaunchKernelGGL(pool_blocks_kernel<bf16_t>, dim3(tokens, kv_heads), dim3(256), (size_t)4 * value_dim * sizeof(float), (hipStream_t)stream, a);
+    hipLaunchKernelGGL(pool_blocks_kernel<bf16_t>, dim3(tokens / pool + batch, kv_heads), dim3(256), (size_t)4 * value_dim * sizeof(float), (hipStream_t)stream, a);
   }
   NNIS_LAUNCH_CHECK("pool_blocks");
   return 0;

@@ -114,7 +114,8 @@ _SUBLAYER_SIGNATURES = {
     "nnis_sigmoid_gate": [_VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_head_norm_write": [_VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID, _VOID, _INT, _FLT, _VOID, _VOID, _INT, _INT, _INT,
                              _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _INT, _INT, _VOID],
-    "nnis_pool_blocks": [_VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_pool_blocks": [_VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _INT,
+                         _VOID],
 }
 
 _LATENT_SIGNATURES = {
@@ -2046,22 +2047,24 @@ def head_norm_write(rows: torch.Tensor, columns, q_out: torch.Tensor, q_weight: 
     return q_out
 
 
-def pool_blocks(k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor, pooled: PooledBlocks, tok_slot: torch.Tensor,
-                tok_pos: torch.Tensor, tokens: int, kv_heads: int, head_dim: int, value_dim: int) -> None:
-    """For every token of the step that completes a block of ``pooled.pool`` tokens of its sequence: the mean of the
-    block's keys and the mean of its values, as the pages hold them, into the block's entry of ``pooled``."""
-    for t, what in ((k_pages, "k_pages"), (v_pages, "v_pages"), (block_table, "block_table"), (tok_slot, "tok_slot"), (tok_pos, "tok_pos")):
+def pool_blocks(k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor, pooled: PooledBlocks, ctx, kv_heads: int,
+                head_dim: int, value_dim: int) -> None:
+    """For every block of ``pooled.pool`` tokens that the step ``ctx`` completes in one of its sequences: the mean of
+    the block's keys and the mean of its values, as the pages hold them, into the block's entry of ``pooled``."""
+    for t, what in ((k_pages, "k_pages"), (v_pages, "v_pages"), (block_table, "block_table")):
         _dev(t, what)
     pooled.check(k_pages, v_pages, kv_heads, head_dim, value_dim, window=1)
     if not _pages_fit(k_pages, v_pages, kv_heads, head_dim, value_dim):
         raise KernelError(f"pool_blocks: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
-    if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or tok_slot.numel() < tokens or tok_pos.numel() < tokens:
-        raise KernelError("pool_blocks: tok_slot / tok_pos must be int32 with one entry per token")
+    _step_arrays(ctx, "pool_blocks")
+    _dev(ctx.seq_pos0, "step metadata")
+    if ctx.seq_pos0.dtype != torch.int32 or ctx.seq_pos0.numel() < ctx.batch:
+        raise KernelError("pool_blocks: the step's first positions must be int32, one a sequence")
     lib = sublayer()
     _check(lib, lib.nnis_pool_blocks(k_pages.data_ptr(), v_pages.data_ptr(), _code(k_pages), block_table.data_ptr(), block_table.shape[1],
                                      pooled.k_pages.data_ptr(), pooled.v_pages.data_ptr(), pooled.block_table.data_ptr(),
-                                     pooled.block_table.shape[1], tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, kv_heads, head_dim,
-                                     int(value_dim), pooled.pool, _stream()))
+                                     pooled.block_table.shape[1], ctx.seq_slot.data_ptr(), ctx.seq_start.data_ptr(),
+                                     ctx.seq_pos0.data_ptr(), ctx.batch, ctx.tokens, kv_heads, head_dim, int(value_dim), pooled.pool, _stream()))
 
 
 def min_gru(rows: torch.Tensor, z_bias: Optional[torch.Tensor], x_bias: Optional[torch.Tensor], state: torch.Tensor, ctx,

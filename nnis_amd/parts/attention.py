@@ -376,8 +376,7 @@ class GatedWindowAttention(Mixer):
         if pooled_view is not None:
             pooled = rt.ops.PooledBlocks(pooled_view.k_pages, pooled_view.v_pages, pooled_view.block_table, self.pool)
             if writes_pooled:
-                rt.ops.pool_blocks(main.k_pages, main.v_pages, main.block_table, pooled, ctx.tok_slot, ctx.tok_pos, tokens,
-                                   self.kv_heads, self.head_dim, self.value_dim)
+                rt.ops.pool_blocks(main.k_pages, main.v_pages, main.block_table, pooled, ctx, self.kv_heads, self.head_dim, self.value_dim)
         plan = None
         if self._matrix_cores(rt) and main.k_pages.dtype == torch.bfloat16:
             plan = (self.decode_plan(ctx.batch, ctx.planned_len, rt) if ctx.decode

@@ -78,7 +78,7 @@ def _run_in_steps(forward, cache, rt, xs, cuts):
 # ---------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("tokens, width", [(1, 8), (37, 50), (5, 1030)])
+@pytest.mark.parametrize("tokens, width", [(1, 8), (37, 50), (5, 1030), (9, 2048), (3, 4096), (2, 4104), (300, 96)])
 def test_the_norm_on_the_way_out(y_dtype, tokens, width):
     from nnis_amd.kernels import ops
 
@@ -106,7 +106,7 @@ def test_the_norm_on_the_way_out(y_dtype, tokens, width):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows, inner", [(1, 8), (33, 72), (4, 1500)])
+@pytest.mark.parametrize("rows, inner", [(1, 8), (33, 72), (4, 1500), (7, 5632), (2, 8192), (3, 8200), (40, 74)])
 def test_poly_norm(dtype, rows, inner):
     from nnis_amd.kernels import ops
 

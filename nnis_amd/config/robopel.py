@@ -71,7 +71,7 @@ class AttentionSizes:
                   _number(raw, "scale", where))
         if out.heads % out.kv_heads:
             raise InvalidInput(f"config.json {where}: {out.heads} heads do not divide into {out.kv_heads} kv_heads")
-        if raw.get("softcap") is not None:
+        if raw.get("softcap") not in (None, 0, 0.0):  # (a cap of zero caps nothing, as a missing one)
             out.softcap = _number(raw, "softcap", where)
         rot = raw.get("rot")
         if rot is not None:
@@ -83,7 +83,7 @@ class AttentionSizes:
         mask = raw.get("mask")
         if mask is not None:
             out.window = _int(mask, "size", where + ".mask")
-            if mask.get("pool") is not None:
+            if mask.get("pool") not in (None, 0):  # (blocks of no tokens are no blocks, as a missing size)
                 out.pool = _int(mask, "pool", where + ".mask")
         if raw.get("kv_from") is not None:
             out.kv_from = _int(raw, "kv_from", where, least=0)

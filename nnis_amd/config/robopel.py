@@ -5,7 +5,7 @@ constant that may differ between models: ``vocab``, ``width``, ``norm.eps``,
 ``embedding.scale`` and ``layers``, each with ``type`` (``attention`` or
 ``mingru``), the mixer's sizes in ``mixer`` and its feed-forward in ``mlp``:
 ``{"kind": "dense", "ff": n}``, ``{"kind": "moe", "expert": {"ff": n},
-"router": {"experts", "top", "identity"}}`` or null for none.  No size has a
+"router": {"experts", "top", "identity"}}`` or null (or absent) for none.  No size has a
 default: a size that is missing is an error, so that a model never runs on a
 guess.  A mechanism that the file does not mention at all does not exist in
 that model: without ``embedding.scale`` rows stay as they are; an attention
@@ -125,7 +125,8 @@ class RobopelConfig:
         out_layers: List[LayerSizes] = []
         for index, layer in enumerate(layers):
             where = f"layers[{index}]"
-            kind, mixer, mlp = _get(layer, "type", where), _get(layer, "mixer", where), _get(layer, "mlp", where)
+            kind, mixer = _get(layer, "type", where), _get(layer, "mixer", where)
+            mlp = layer.get("mlp") if isinstance(layer, dict) else None  # (absent or null: the layer has no feed-forward)
             if kind == "attention":
                 sizes = LayerSizes(kind, attention=AttentionSizes.from_dict(mixer, where + ".mixer"))
                 source = sizes.attention.kv_from

@@ -52,7 +52,7 @@ def test_layers_their_parts_and_whose_keys_they_read():
 def test_missing_and_wrong_keys_are_refused():
     for path in (["vocab"], ["norm", "eps"], ["layers", 0, "mixer", "heads"], ["layers", 0, "mixer", "scale"], ["layers", 0, "mixer", "vdim"],
                  ["layers", 0, "mixer", "rot", "base"], ["layers", 0, "mixer", "rot", "scaling", "low"], ["layers", 0, "mixer", "mask", "size"],
-                 ["layers", 0, "mlp"], ["layers", 0, "mlp", "ff"], ["layers", 1, "mixer", "width"], ["layers", 1, "mlp", "router", "top"],
+                 ["layers", 0, "mlp", "ff"], ["layers", 1, "mixer", "width"], ["layers", 1, "mlp", "router", "top"],
                  ["layers", 1, "mlp", "expert"]):
         raw = copy.deepcopy(ROB_A)
         at = raw
@@ -84,6 +84,10 @@ def test_missing_and_wrong_keys_are_refused():
 
 
 def test_what_the_file_does_not_mention_does_not_exist():
+    bare = robopel(vocab=50, width=32, layers=[{"type": "mingru", "mixer": {"width": 8}}])  # no "mlp" at all: no feed-forward
+    assert "feed_forward" not in spec_from_config(bare)[1].layers[0]
+    zeros = robopel(vocab=50, width=32, layers=[layer("attention", dict(attention(2, 1, 16, 8, window=5), softcap=0, mask={"size": 5, "pool": 0}))])
+    assert (spec_from_config(zeros)[0].layers[0].attention.softcap, spec_from_config(zeros)[0].layers[0].attention.pool) == (0.0, 0)
     config = robopel(vocab=50, width=32, layers=[layer("attention", attention(2, 1, 16, 8, scale=0.3), moe(3, 2, 8))])
     cfg, spec = spec_from_config(config)
     sizes = cfg.layers[0].attention

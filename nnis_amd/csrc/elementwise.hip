@@ -302,6 +302,7 @@ struct RopeWriteArgs {
   int value_dim;     // channels of a value head (head_dim unless the values have a size of their own)
   const void* bias;  // [(heads + kv_heads) * head_dim + kv_heads * value_dim] added before the rotation, or null
   int bias_dtype;
+  int values_from_keys;  // 1: the rows hold no values; a head's value is its key as projected, before the rotation
 };
 
 __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
@@ -312,7 +313,7 @@ __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
   const int hd = a.head_dim;
   const int vd = a.value_dim;
   const int half = a.rot_dim / 2;
-  const int row_width = (a.heads + a.kv_heads) * hd + a.kv_heads * vd;
+  const int row_width = (a.heads + a.kv_heads) * hd + (a.values_from_keys ? 0 : a.kv_heads * vd);
   const size_t in_base = (size_t)token * row_width;
   // element `at` of the token's row, with its bias
   auto element = [&](size_t at) {
@@ -365,7 +366,7 @@ __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
   }
   // values: copied into the page's order
   if (page >= 0) {
-    const size_t v_src = (size_t)(a.heads + a.kv_heads) * hd;
+    const size_t v_src = (size_t)(a.values_from_keys ? a.heads : a.heads + a.kv_heads) * hd;
     for (int item = threadIdx.x; item < a.kv_heads * vd; item += blockDim.x) {
       const int kv_head = item / vd;
       const int d = item % vd;
@@ -386,7 +387,7 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
   const int hd = a.head_dim;
   const int vd = a.value_dim;
   const int half = a.rot_dim / 2;
-  const int row_width = (a.heads + a.kv_heads) * hd + a.kv_heads * vd;
+  const int row_width = (a.heads + a.kv_heads) * hd + (a.values_from_keys ? 0 : a.kv_heads * vd);
   const bf16_t* src = (const bf16_t*)a.qkv + (size_t)token * row_width;
   const bf16_t* bias = (const bf16_t*)a.bias;  // bfloat16 here, or null
   // 4 channels from column `at` of the token's row, with their bias, in 32-bit
@@ -449,7 +450,7 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
       const int v_item = item - rot_items;
       const int kv_head = v_item / (vd / 4);
       const int d = (v_item % (vd / 4)) * 4;
-      const f32x4_t v = four((size_t)(a.heads + a.kv_heads) * hd + (size_t)kv_head * vd + d);
+      const f32x4_t v = four((size_t)(a.values_from_keys ? a.heads : a.heads + a.kv_heads) * hd + (size_t)kv_head * vd + d);
       bf16_t* dst = (bf16_t*)a.v_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(vd);
 #pragma unroll
       for (int j = 0; j < 4; ++j) dst[nnis_v_offset(d + j, in_page)] = (__bf16)v[j];
@@ -458,12 +459,15 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
 }
 
 // value_dim: channels of a value head (0: head_dim); bias: one entry per column of qkv, added before the rotation, or null
-extern "C" int nnis_rope_kv_write_wide(const void* qkv, int qkv_dtype, void* q_out, int q_dtype, const float* cos_table,
-                                       const float* sin_table, int table_positions, int rot_dim, const int* tok_slot,
-                                       const int* tok_pos, void* k_pages, void* v_pages, int cache_dtype,
-                                       const int* block_table, int max_pages, int tokens, int heads, int kv_heads,
-                                       int head_dim, int value_dim, const void* bias, int bias_dtype, void* stream) {
+// values_from_keys: the rows are [q heads | k heads] only, and a head's value is its key as projected (not rotated)
+extern "C" int nnis_rope_kv_write_shared(const void* qkv, int qkv_dtype, void* q_out, int q_dtype, const float* cos_table,
+                                         const float* sin_table, int table_positions, int rot_dim, const int* tok_slot,
+                                         const int* tok_pos, void* k_pages, void* v_pages, int cache_dtype,
+                                         const int* block_table, int max_pages, int tokens, int heads, int kv_heads,
+                                         int head_dim, int value_dim, const void* bias, int bias_dtype, int values_from_keys,
+                                         void* stream) {
   if (value_dim <= 0) value_dim = head_dim;
+  NNIS_REQUIRE(!values_from_keys || value_dim == head_dim, "rope_kv_write: values that are the keys have their size, not %d", value_dim);
   NNIS_REQUIRE(bias == nullptr || nnis_dtype_ok(bias_dtype), "rope_kv_write: unknown bias dtype %d", bias_dtype);
   NNIS_REQUIRE(nnis_dtype_ok(qkv_dtype) && nnis_dtype_ok(q_dtype), "rope_kv_write: unknown dtype");
   NNIS_REQUIRE(k_pages == nullptr || nnis_dtype_ok(cache_dtype), "rope_kv_write: unknown cache dtype %d", cache_dtype);
@@ -481,7 +485,7 @@ extern "C" int nnis_rope_kv_write_wide(const void* qkv, int qkv_dtype, void* q_o
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.k_pages = k_pages; a.v_pages = v_pages;
   a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
   a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
-  a.value_dim = value_dim; a.bias = bias; a.bias_dtype = bias_dtype;
+  a.value_dim = value_dim; a.bias = bias; a.bias_dtype = bias_dtype; a.values_from_keys = values_from_keys ? 1 : 0;
   const bool all_bf16 = qkv_dtype == NNIS_BF16 && q_dtype == NNIS_BF16 && (k_pages == nullptr || cache_dtype == NNIS_BF16);
   const bool aligned = ((uintptr_t)qkv % 16 == 0) && ((uintptr_t)q_out % 16 == 0) && ((uintptr_t)k_pages % 16 == 0) &&
                        ((uintptr_t)v_pages % 16 == 0) && ((uintptr_t)cos_table % 16 == 0) && ((uintptr_t)sin_table % 16 == 0);
@@ -498,6 +502,16 @@ extern "C" int nnis_rope_kv_write_wide(const void* qkv, int qkv_dtype, void* q_o
   hipLaunchKernelGGL(rope_kv_write_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
   NNIS_LAUNCH_CHECK("rope_kv_write");
   return 0;
+}
+
+extern "C" int nnis_rope_kv_write_wide(const void* qkv, int qkv_dtype, void* q_out, int q_dtype, const float* cos_table,
+                                       const float* sin_table, int table_positions, int rot_dim, const int* tok_slot,
+                                       const int* tok_pos, void* k_pages, void* v_pages, int cache_dtype,
+                                       const int* block_table, int max_pages, int tokens, int heads, int kv_heads,
+                                       int head_dim, int value_dim, const void* bias, int bias_dtype, void* stream) {
+  return nnis_rope_kv_write_shared(qkv, qkv_dtype, q_out, q_dtype, cos_table, sin_table, table_positions, rot_dim, tok_slot, tok_pos,
+                                   k_pages, v_pages, cache_dtype, block_table, max_pages, tokens, heads, kv_heads, head_dim, value_dim,
+                                   bias, bias_dtype, 0, stream);
 }
 
 extern "C" int nnis_rope_kv_write(const void* qkv, int qkv_dtype, void* q_out, int q_dtype, const float* cos_table,

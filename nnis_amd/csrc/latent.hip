@@ -104,20 +104,65 @@ __global__ void latent_rotate_q_kernel(void* __restrict__ q, int q_dtype, int he
   }
 }
 
-__global__ void head_scale_kernel(void* __restrict__ o, int o_dtype, const float* __restrict__ gate, int channels, size_t total) {
+// logistic: the gates are logits still, and a head is multiplied by 1 / (1 + exp(-gate))
+__device__ __forceinline__ float head_gate_of(float g, int logistic) { return logistic ? 1.0f / (1.0f + expf(-g)) : g; }
+
+__global__ void head_scale_kernel(void* __restrict__ o, int o_dtype, const float* __restrict__ gate, int channels, size_t total,
+                                  int logistic) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
-    store_from_f32(o, o_dtype, i, load_as_f32(o, o_dtype, i) * gate[i / channels]);
+    store_from_f32(o, o_dtype, i, load_as_f32(o, o_dtype, i) * head_gate_of(gate[i / channels], logistic));
 }
 
 // the same on bfloat16 rows whose heads come in steps of 8 channels: 16-byte accesses
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_l;
-__global__ void head_scale_bf16_kernel(bf16_t* __restrict__ o, const float* __restrict__ gate, int channels, size_t groups) {
+__global__ void head_scale_bf16_kernel(bf16_t* __restrict__ o, const float* __restrict__ gate, int channels, size_t groups, int logistic) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < groups; i += (size_t)gridDim.x * blockDim.x) {
-    const float g = gate[(i * 8) / channels];
+    const float g = head_gate_of(gate[(i * 8) / channels], logistic);
     bf16x8_l v = *(const bf16x8_l*)(o + i * 8);
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * g);
     *(bf16x8_l*)(o + i * 8) = v;
+  }
+}
+
+// -----------------------------------------------------------------------------
+// A map of their own for every head: out[t, h, n] = (sum_k w[h, n, k] x[t, h, k]) * gate[t, h * N + n], x [tokens,
+// heads * K], w [heads, N, K], gate (32-bit, optional) [tokens, heads * N].  The heads' value maps of attention over
+// a latent where a gate element by element stands between them and the output projection, so that they cannot be
+// folded into it.  A block takes R rows of one head, kept in LDS as floats; a wave takes an output at a time for all
+// of them (lanes stride over k), so a row of the head's map is read once a block.  Sums are 32-bit.
+// -----------------------------------------------------------------------------
+template <int R>
+__global__ __launch_bounds__(256) void heads_linear_kernel(const void* __restrict__ x, int x_dtype, const void* __restrict__ w, int w_dtype,
+                                                           const float* __restrict__ gate, void* __restrict__ out, int out_dtype,
+                                                           int tokens, int heads, int n, int k) {
+  extern __shared__ __attribute__((aligned(16))) float xs[];  // [R][k]
+  const int head = blockIdx.y, row0 = blockIdx.x * R;
+  for (int i = threadIdx.x; i < R * k; i += blockDim.x) {
+    const int r = i / k;
+    xs[i] = row0 + r < tokens ? load_as_f32(x, x_dtype, ((size_t)(row0 + r) * heads + head) * k + i % k) : 0.0f;
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, waves = blockDim.x / kWave;
+  for (int o = wave; o < n; o += waves) {
+    const size_t w_row = ((size_t)head * n + o) * k;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+#pragma unroll 4
+    for (int c = lane; c < k; c += kWave) {
+      const float wv = load_as_f32(w, w_dtype, w_row + c);
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] = fmaf(xs[r * k + c], wv, acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float total = wave_sum(acc[r]);
+      if (lane == 0 && row0 + r < tokens) {
+        const size_t at = ((size_t)(row0 + r) * heads + head) * n + o;
+        store_from_f32(out, out_dtype, at, gate ? total * gate[at] : total);
+      }
+    }
   }
 }
 
@@ -171,18 +216,43 @@ extern "C" int nnis_latent_rotate_q(void* q, int q_dtype, int tokens, int heads,
   return 0;
 }
 
+extern "C" int nnis_head_scale_of(void* o, int o_dtype, const float* gate, int tokens, int heads, int channels, int logistic, void* stream);
+
 extern "C" int nnis_head_scale(void* o, int o_dtype, const float* gate, int tokens, int heads, int channels, void* stream) {
+  return nnis_head_scale_of(o, o_dtype, gate, tokens, heads, channels, 0, stream);
+}
+
+// logistic: gate holds logits, and head h of token t is multiplied by sigmoid(gate[t, h])
+extern "C" int nnis_head_scale_of(void* o, int o_dtype, const float* gate, int tokens, int heads, int channels, int logistic, void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(o_dtype), "head_scale: unknown dtype");
   NNIS_REQUIRE(o && gate && tokens >= 0 && heads > 0 && channels > 0, "head_scale: bad arguments");
   if (tokens == 0) return 0;
   const size_t total = (size_t)tokens * heads * channels;
   if (o_dtype == NNIS_BF16 && channels % 8 == 0 && (uintptr_t)o % 16 == 0) {
     hipLaunchKernelGGL(head_scale_bf16_kernel, dim3(blocks_for(total / 8)), dim3(256), 0, (hipStream_t)stream, (bf16_t*)o, gate, channels,
-                       total / 8);
+                       total / 8, logistic);
     NNIS_LAUNCH_CHECK("head_scale");
     return 0;
   }
-  hipLaunchKernelGGL(head_scale_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, o, o_dtype, gate, channels, total);
+  hipLaunchKernelGGL(head_scale_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, o, o_dtype, gate, channels, total, logistic);
   NNIS_LAUNCH_CHECK("head_scale");
+  return 0;
+}
+
+extern "C" int nnis_heads_linear(const void* x, int x_dtype, const void* w, int w_dtype, const float* gate, void* out, int out_dtype,
+                                 int tokens, int heads, int n, int k, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(x_dtype) && nnis_dtype_ok(w_dtype) && nnis_dtype_ok(out_dtype), "heads_linear: unknown dtype");
+  NNIS_REQUIRE(x && w && out && tokens >= 0 && heads > 0 && heads <= 65535 && n > 0 && k > 0, "heads_linear: bad arguments");
+  NNIS_REQUIRE((size_t)k * sizeof(float) <= 48 * 1024, "heads_linear: rows of up to 12288 channels a head, got %d", k);
+  if (tokens == 0) return 0;
+  // several rows a block where they fit 48 KB of LDS and the step has rows enough
+  const int rows = tokens >= 64 && (size_t)8 * k * 4 <= 49152 ? 8 : (tokens >= 4 && (size_t)4 * k * 4 <= 49152 ? 4 : 1);
+  const dim3 grid((tokens + rows - 1) / rows, heads);
+  const size_t lds = (size_t)rows * k * sizeof(float);
+  hipStream_t s = (hipStream_t)stream;
+  if (rows == 8) hipLaunchKernelGGL((heads_linear_kernel<8>), grid, dim3(256), lds, s, x, x_dtype, w, w_dtype, gate, out, out_dtype, tokens, heads, n, k);
+  else if (rows == 4) hipLaunchKernelGGL((heads_linear_kernel<4>), grid, dim3(256), lds, s, x, x_dtype, w, w_dtype, gate, out, out_dtype, tokens, heads, n, k);
+  else hipLaunchKernelGGL((heads_linear_kernel<1>), grid, dim3(256), lds, s, x, x_dtype, w, w_dtype, gate, out, out_dtype, tokens, heads, n, k);
+  NNIS_LAUNCH_CHECK("heads_linear");
   return 0;
 }

@@ -374,7 +374,31 @@ struct GlaArgs {
   int piece, pieces;
   float* carried;  // [batch, pieces, heads, key_dim, value_dim]
   float* decayed;  // [batch, pieces, heads, key_dim]: a piece's sum of the decays' logarithms
+  // Without `zd`: one fixed decay a head (retention), head_decay [2, heads]: the decays, then their logarithms.
+  const float* head_decay;
+  // With rot_dim > 0: the first rot_dim channels of every head of q and k are turned by the token's position while
+  // they are staged, channel i with channel i + rot_dim / 2: (u, v) -> (u cos - v sin, v cos + u sin), tables
+  // [rot_positions, rot_dim / 2], tok_pos one position a row of the step.
+  const float* rot_cos;
+  const float* rot_sin;
+  const int* tok_pos;
+  int rot_dim, rot_positions;
 };
+
+// channel `ch` of head `head` of row t, turned by the row's position where the head's first channels are
+__device__ __forceinline__ float gla_turned(const GlaArgs& a, const void* base, int stride, int t, int head, int ch) {
+  const size_t row = (size_t)t * stride + (size_t)head * a.key_dim;
+  const float x = load_as_f32(base, a.qkv_dtype, row + ch);
+  if (ch >= a.rot_dim) return x;
+  const int half = a.rot_dim / 2;
+  const bool low = ch < half;
+  const int pair = low ? ch : ch - half;
+  int pos = a.tok_pos[t];
+  pos = pos < 0 ? 0 : (pos < a.rot_positions ? pos : a.rot_positions - 1);
+  const float c = a.rot_cos[(size_t)pos * half + pair], s = a.rot_sin[(size_t)pos * half + pair];
+  const float other = load_as_f32(base, a.qkv_dtype, row + (low ? ch + half : ch - half));
+  return low ? x * c - other * s : x * c + other * s;
+}
 
 // PASS as in selective_scan_kernel: 0 a whole run; 1 a piece from a zero state, leaving its end and the sum of its
 // decays' logarithms; 3 a piece from the state that the carry kernel left for it, writing the outputs.
@@ -428,16 +452,20 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
     __syncthreads();  // the chunk before has been read
     for (int i = threadIdx.x; i < count * d; i += blockDim.x) {
       const int t = t0 + i / d, ch = i % d;
-      if (PASS != 1) qs[i] = load_as_f32(a.q, a.qkv_dtype, (size_t)t * a.q_stride + head * d + ch) * a.scale;
-      ks[i] = load_as_f32(a.k, a.qkv_dtype, (size_t)t * a.k_stride + head * d + ch);
-      as[i] = exp2_fast(a.zd[((size_t)t * a.heads + head) * d + ch] * kLog2e);
+      if (PASS != 1) qs[i] = gla_turned(a, a.q, a.q_stride, t, head, ch) * a.scale;
+      ks[i] = gla_turned(a, a.k, a.k_stride, t, head, ch);
+      as[i] = a.zd ? exp2_fast(a.zd[((size_t)t * a.heads + head) * d + ch] * kLog2e) : a.head_decay[head];
     }
     for (int i = threadIdx.x; i < count * kCols; i += blockDim.x) {
       const int t = t0 + i / kCols, cl = blockIdx.x * kCols + i % kCols;
       vs[i] = cl < e ? load_as_f32(a.v, a.qkv_dtype, (size_t)t * a.v_stride + head * e + cl) : 0.0f;
     }
     if (PASS == 1 && blockIdx.x == 0 && (int)threadIdx.x < d) {
-      for (int j = 0; j < count; ++j) log_sum += a.zd[((size_t)(t0 + j) * a.heads + head) * d + threadIdx.x];
+      if (a.zd) {
+        for (int j = 0; j < count; ++j) log_sum += a.zd[((size_t)(t0 + j) * a.heads + head) * d + threadIdx.x];
+      } else {
+        log_sum += (float)count * a.head_decay[a.heads + head];
+      }
     }
     __syncthreads();
     for (int j = 0; j < count; ++j) {
@@ -553,7 +581,7 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   const float scale = 1.0f / sqrtf(wave_sum(squares) / (float)dim + eps);
   for (int c = lane; c < dim; c += kWave) {
     const float g = load_as_f32(gate, gate_dtype, (size_t)token * gate_stride + head * dim + c);
-    const float v = (row[c] * scale) * load_as_f32(weight, weight_dtype, c);
+    const float v = (row[c] * scale) * (weight ? load_as_f32(weight, weight_dtype, c) : 1.0f);
     store_from_f32(y, y_dtype, (size_t)item * dim + c, v * (g * sigmoid_f(g)));
   }
 }
@@ -636,14 +664,35 @@ extern "C" int nnis_selective_scan(const void* x, int x_dtype, const float* dt_p
 
 // piece, pieces: as nnis_selective_scan's (`carried`: batch * pieces * heads * key_dim * value_dim floats, `decayed`:
 // batch * pieces * heads * key_dim)
+// Without `zd`: `head_decay` [2, heads], one fixed decay a head and its logarithm.  rot_dim > 0: q's and k's first
+// rot_dim channels of a head are turned by tok_pos[row] while staged (tables [rot_positions, rot_dim / 2]).
+extern "C" int nnis_gla_scan_turned(const void* q, const void* k, const void* v, int qkv_dtype, int q_stride, int k_stride, int v_stride,
+                                    const float* zd, const float* head_decay, const float* rot_cos, const float* rot_sin,
+                                    int rot_dim, int rot_positions, const int* tok_pos, float scale, float* state,
+                                    const int* seq_slot, const int* seq_start, int batch, int heads, int key_dim, int value_dim,
+                                    float* out, int piece, int pieces, float* carried, float* decayed, void* stream);
+
 extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qkv_dtype, int q_stride, int k_stride, int v_stride,
                              const float* zd, float scale, float* state, const int* seq_slot, const int* seq_start,
                              int batch, int heads, int key_dim, int value_dim, float* out, int piece, int pieces, float* carried,
                              float* decayed, void* stream) {
+  NNIS_REQUIRE(zd, "gla_scan: the decays' logarithms are missing");
+  return nnis_gla_scan_turned(q, k, v, qkv_dtype, q_stride, k_stride, v_stride, zd, nullptr, nullptr, nullptr, 0, 0, nullptr, scale,
+                              state, seq_slot, seq_start, batch, heads, key_dim, value_dim, out, piece, pieces, carried, decayed, stream);
+}
+
+extern "C" int nnis_gla_scan_turned(const void* q, const void* k, const void* v, int qkv_dtype, int q_stride, int k_stride, int v_stride,
+                                    const float* zd, const float* head_decay, const float* rot_cos, const float* rot_sin,
+                                    int rot_dim, int rot_positions, const int* tok_pos, float scale, float* state,
+                                    const int* seq_slot, const int* seq_start, int batch, int heads, int key_dim, int value_dim,
+                                    float* out, int piece, int pieces, float* carried, float* decayed, void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(qkv_dtype), "gla_scan: unknown dtype %d", qkv_dtype);
+  NNIS_REQUIRE((zd != nullptr) != (head_decay != nullptr), "gla_scan: decays a token and channel, or one a head");
+  NNIS_REQUIRE(rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= key_dim, "gla_scan: %d turned channels in heads of %d", rot_dim, key_dim);
+  NNIS_REQUIRE(rot_dim == 0 || (rot_cos && rot_sin && tok_pos && rot_positions > 0), "gla_scan: a rotation needs tables and positions");
   NNIS_REQUIRE(heads > 0 && key_dim > 0 && key_dim <= 256 && value_dim > 0 && batch >= 0,
                "gla_scan: bad sizes (heads %d, key channels %d: up to 256 are taken, value channels %d)", heads, key_dim, value_dim);
-  NNIS_REQUIRE(q && k && v && zd && state && seq_slot && seq_start && out, "gla_scan: a pointer is missing");
+  NNIS_REQUIRE(q && k && v && state && seq_slot && seq_start && out, "gla_scan: a pointer is missing");
   NNIS_REQUIRE(pieces <= 1 || (piece > 0 && carried && decayed), "gla_scan: pieces need their length and scratch");
   if (pieces < 1) pieces = 1;
   NNIS_REQUIRE((long long)batch * pieces <= 65535 && heads <= 65535, "gla_scan: %d sequences x %d pieces exceed the grid limit", batch, pieces);
@@ -652,6 +701,7 @@ extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qk
   a.q = q; a.k = k; a.v = v; a.qkv_dtype = qkv_dtype; a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.zd = zd;
   a.scale = scale; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.heads = heads;
   a.key_dim = key_dim; a.value_dim = value_dim; a.out = out; a.piece = piece; a.pieces = pieces; a.carried = carried; a.decayed = decayed;
+  a.head_decay = head_decay; a.rot_cos = rot_cos; a.rot_sin = rot_sin; a.tok_pos = tok_pos; a.rot_dim = rot_dim; a.rot_positions = rot_positions;
   const int need = (key_dim + 15) / 16;
   const int groups = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : (need <= 8 ? 8 : 16)));
   const int span = 4 * (kWave / groups);
@@ -715,9 +765,9 @@ extern "C" int nnis_gla_decays(float* z, const float* bias, int tokens, int widt
 
 extern "C" int nnis_head_norm_gate(const float* o, const void* gate, int gate_dtype, int gate_stride, const void* weight,
                                    int weight_dtype, void* y, int y_dtype, int tokens, int heads, int dim, float eps, void* stream) {
-  NNIS_REQUIRE(nnis_dtype_ok(gate_dtype) && nnis_dtype_ok(weight_dtype) && nnis_dtype_ok(y_dtype), "head_norm_gate: unknown dtype");
+  NNIS_REQUIRE(nnis_dtype_ok(gate_dtype) && (!weight || nnis_dtype_ok(weight_dtype)) && nnis_dtype_ok(y_dtype), "head_norm_gate: unknown dtype");
   NNIS_REQUIRE(tokens >= 0 && heads > 0 && dim > 0 && gate_stride >= heads * dim && eps > 0.0f, "head_norm_gate: bad sizes");
-  NNIS_REQUIRE(o && gate && weight && y, "head_norm_gate: a pointer is missing");
+  NNIS_REQUIRE(o && gate && y, "head_norm_gate: a pointer is missing");
   const int items = tokens * heads;
   if (items == 0) return 0;
   hipLaunchKernelGGL(head_norm_gate_kernel, dim3((items + 3) / 4), dim3(256), 0, (hipStream_t)stream, o, gate, gate_dtype, gate_stride,
@@ -836,5 +886,180 @@ extern "C" int nnis_min_gru(const void* rows, int dtype, int stride, const void*
   }
   hipLaunchKernelGGL(min_gru_kernel<2>, grid, dim3(threads), 0, (hipStream_t)stream, a);
   NNIS_LAUNCH_CHECK("min_gru");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// Gated delta rule.  Per head, over a sequence's tokens, with a state S [key channels, value channels]:
+//   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+// with q and k unit vectors over a head's channels (x / sqrt(sum x^2 + unit_eps); q also times q_scale), beta =
+// sigmoid(b), g = exp(-rate_h * softplus(a + dt_bias_h)).  Query/key head of value head h: h / (heads / groups).
+// The columns of S do not meet: a block takes one head of one sequence and a slab of value columns; a thread keeps
+// 16 key rows of one column, the threads of a column sit 64 / GROUPS lanes apart in one wave and add their parts of
+// S^T k and S^T q by lane exchanges.  Tokens come through LDS a chunk at a time: a wave a token makes the unit
+// vectors, a thread a token the gates.  Everything but the rows' storage type is 32-bit; o is left raw, in 32-bit.
+// -----------------------------------------------------------------------------
+namespace {
+
+struct DeltaArgs {
+  const void* rows;  // row t: [q (groups * key_dim) | k (groups * key_dim) | v (heads * value_dim)]
+  int dtype, stride;
+  const float* ba;  // [tokens, 2 * heads]: b of every head, then a
+  const float* rate;     // [heads]: exp(A_log)
+  const float* dt_bias;  // [heads]
+  float q_scale, unit_eps;
+  float* state;  // [slots, heads, key_dim, value_dim]
+  const int* seq_slot;
+  const int* seq_start;
+  int heads, groups, key_dim, value_dim;
+  int chunk;
+  float* out;  // [tokens, heads * value_dim]
+};
+
+template <int GROUPS>
+__global__ __launch_bounds__(256) void gated_delta_kernel(DeltaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  constexpr int kPad = GROUPS * 16;            // key rows as the threads see them (rows beyond key_dim are zero)
+  constexpr int kPer = kWave / GROUPS;         // columns of a wave
+  constexpr int kCols = 4 * kPer;              // columns of a block
+  constexpr int kEach = (kPad + kWave - 1) / kWave;  // channels a lane takes of a vector
+  const int b = blockIdx.z, head = blockIdx.y;
+  const int slot = a.seq_slot[b];
+  if (slot < 0) return;
+  const int begin = a.seq_start[b], end = a.seq_start[b + 1];
+  if (end <= begin) return;
+  const int d = a.key_dim, e = a.value_dim;
+  const int qk_head = head / (a.heads / a.groups);
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int group = lane / kPer;
+  const int col_in_block = wave * kPer + lane % kPer;
+  const int col = blockIdx.x * kCols + col_in_block;
+  const bool live = col < e;
+  float* qs = lds;                     // [chunk][kPad]
+  float* ks = qs + a.chunk * kPad;     // [chunk][kPad]
+  float* vs = ks + a.chunk * kPad;     // [chunk][kCols]
+  float* gs = vs + a.chunk * kCols;    // [chunk][2]: g, beta
+  float* state = a.state + (((size_t)slot * a.heads + head) * d) * e + (live ? col : 0);
+  float S[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = group * 16 + r;
+    S[r] = live && row < d ? state[(size_t)row * e] : 0.0f;
+  }
+  const size_t k_col0 = (size_t)a.groups * d;
+  const size_t v_col0 = 2 * (size_t)a.groups * d;
+  for (int t0 = begin; t0 < end; t0 += a.chunk) {
+    const int count = min(a.chunk, end - t0);
+    __syncthreads();  // the chunk before has been read
+    // unit vectors: a wave a (token, query or key)
+    for (int item = wave; item < 2 * count; item += 4) {
+      const int j = item >> 1, is_key = item & 1;
+      const size_t at = (size_t)(t0 + j) * a.stride + (is_key ? k_col0 : 0) + (size_t)qk_head * d;
+      float x[kEach];
+      float ss = 0.0f;
+#pragma unroll
+      for (int i = 0; i < kEach; ++i) {
+        const int ch = i * kWave + lane;
+        x[i] = ch < d ? load_as_f32(a.rows, a.dtype, at + ch) : 0.0f;
+        ss = fmaf(x[i], x[i], ss);
+      }
+      const float inv = (1.0f / sqrtf(wave_sum(ss) + a.unit_eps)) * (is_key ? 1.0f : a.q_scale);
+      float* into = (is_key ? ks : qs) + j * kPad;
+#pragma unroll
+      for (int i = 0; i < kEach; ++i) {
+        const int ch = i * kWave + lane;
+        if (ch < kPad) into[ch] = x[i] * inv;
+      }
+    }
+    for (int i = threadIdx.x; i < count * kCols; i += blockDim.x) {
+      const int t = t0 + i / kCols, cl = blockIdx.x * kCols + i % kCols;
+      vs[i] = cl < e ? load_as_f32(a.rows, a.dtype, (size_t)t * a.stride + v_col0 + (size_t)head * e + cl) : 0.0f;
+    }
+    if ((int)threadIdx.x < count) {
+      const float* ba = a.ba + (size_t)(t0 + threadIdx.x) * 2 * a.heads;
+      const float z = ba[a.heads + head] + a.dt_bias[head];
+      const float soft = z > 20.0f ? z : log1pf(expf(z));
+      gs[2 * threadIdx.x] = expf(-a.rate[head] * soft);
+      gs[2 * threadIdx.x + 1] = 1.0f / (1.0f + expf(-ba[head]));
+    }
+    __syncthreads();
+    for (int j = 0; j < count; ++j) {
+      const float g = gs[2 * j], beta = gs[2 * j + 1];
+      const float v = vs[j * kCols + col_in_block];
+      const float* qj = qs + j * kPad + group * 16;
+      const float* kj = ks + j * kPad + group * 16;
+      float kv[16];
+      float dot = 0.0f;
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const float4 k4 = *(const float4*)(kj + 4 * r4);
+        kv[4 * r4] = k4.x; kv[4 * r4 + 1] = k4.y; kv[4 * r4 + 2] = k4.z; kv[4 * r4 + 3] = k4.w;
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        S[r] *= g;
+        dot = fmaf(S[r], kv[r], dot);
+      }
+#pragma unroll
+      for (int offset = kWave / 2; offset >= kPer; offset >>= 1) dot += __shfl_xor(dot, offset, kWave);
+      const float u = beta * (v - dot);
+      float acc = 0.0f;
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const float4 q4 = *(const float4*)(qj + 4 * r4);
+        const float qv[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          S[4 * r4 + i] = fmaf(kv[4 * r4 + i], u, S[4 * r4 + i]);
+          acc = fmaf(S[4 * r4 + i], qv[i], acc);
+        }
+      }
+#pragma unroll
+      for (int offset = kWave / 2; offset >= kPer; offset >>= 1) acc += __shfl_xor(acc, offset, kWave);
+      if (group == 0 && live) a.out[((size_t)(t0 + j) * a.heads + head) * e + col] = acc;
+    }
+  }
+  if (!live) return;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = group * 16 + r;
+    if (row < d) state[(size_t)row * e] = S[r];
+  }
+}
+
+}  // namespace
+
+// rows [tokens, stride] hold [q | k | v] behind the convolution; ba float32 [tokens, 2 * heads]; out float32 [tokens, heads * value_dim]
+extern "C" int nnis_gated_delta(const void* rows, int dtype, int stride, const float* ba, const float* rate, const float* dt_bias,
+                                float q_scale, float unit_eps, float* state, const int* seq_slot, const int* seq_start, int batch,
+                                int heads, int groups, int key_dim, int value_dim, float* out, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(dtype), "gated_delta: unknown dtype %d", dtype);
+  NNIS_REQUIRE(heads > 0 && groups > 0 && heads % groups == 0 && key_dim > 0 && key_dim <= 256 && value_dim > 0 && batch >= 0,
+               "gated_delta: bad sizes (heads %d on %d query/key heads, key channels %d: up to 256 are taken, value channels %d)", heads,
+               groups, key_dim, value_dim);
+  NNIS_REQUIRE(stride >= 2 * groups * key_dim + heads * value_dim, "gated_delta: rows of %d are too short", stride);
+  NNIS_REQUIRE(rows && ba && rate && dt_bias && state && seq_slot && seq_start && out, "gated_delta: a pointer is missing");
+  NNIS_REQUIRE(batch <= 65535 && heads <= 65535, "gated_delta: %d sequences exceed the grid limit", batch);
+  if (batch == 0) return 0;
+  DeltaArgs a;
+  a.rows = rows; a.dtype = dtype; a.stride = stride; a.ba = ba; a.rate = rate; a.dt_bias = dt_bias; a.q_scale = q_scale;
+  a.unit_eps = unit_eps; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.heads = heads; a.groups = groups;
+  a.key_dim = key_dim; a.value_dim = value_dim; a.out = out;
+  const int need = (key_dim + 15) / 16;
+  const int lane_groups = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : (need <= 8 ? 8 : 16)));
+  const int cols = 4 * (kWave / lane_groups);
+  const int pad = lane_groups * 16;
+  a.chunk = 16;
+  const size_t lds = (size_t)a.chunk * (2 * pad + cols + 2) * sizeof(float);
+  const dim3 grid((value_dim + cols - 1) / cols, heads, batch);
+  hipStream_t s = (hipStream_t)stream;
+  switch (lane_groups) {
+    case 1: hipLaunchKernelGGL(gated_delta_kernel<1>, grid, dim3(256), lds, s, a); break;
+    case 2: hipLaunchKernelGGL(gated_delta_kernel<2>, grid, dim3(256), lds, s, a); break;
+    case 4: hipLaunchKernelGGL(gated_delta_kernel<4>, grid, dim3(256), lds, s, a); break;
+    case 8: hipLaunchKernelGGL(gated_delta_kernel<8>, grid, dim3(256), lds, s, a); break;
+    default: hipLaunchKernelGGL(gated_delta_kernel<16>, grid, dim3(256), lds, s, a); break;
+  }
+  NNIS_LAUNCH_CHECK("gated_delta");
   return 0;
 }

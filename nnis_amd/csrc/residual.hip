@@ -670,3 +670,63 @@ extern "C" int nnis_tanh_cap(float* x, float cap, long long total, void* stream)
   NNIS_LAUNCH_CHECK("tanh_cap");
   return 0;
 }
+
+// -----------------------------------------------------------------------------
+// Branches side by side, plainly: out = sum_i scale_i * y_i, the sum in 32-bit.  Up to kMostBranches inputs of one
+// type and shape, each with a factor.
+// -----------------------------------------------------------------------------
+struct BranchSumArgs {
+  const void* y[kMostBranches];
+  float scale[kMostBranches];
+  int count;
+  int y_dtype;
+  void* out;
+  int out_dtype;
+  size_t total;
+};
+
+__global__ void branch_sum_kernel(BranchSumArgs a) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.total; i += (size_t)gridDim.x * blockDim.x) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int b = 0; b < kMostBranches; ++b)
+      if (b < a.count) sum = fmaf(a.scale[b], load_as_f32(a.y[b], a.y_dtype, i), sum);
+    store_from_f32(a.out, a.out_dtype, i, sum);
+  }
+}
+
+extern "C" int nnis_branch_sum(const void* const* y, const float* scale, int count, int y_dtype, long long total, void* out, int out_dtype,
+                               void* stream) {
+  NNIS_REQUIRE(count >= 1 && count <= kMostBranches, "branch_sum: 1 to %d branches are taken, got %d", kMostBranches, count);
+  NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(out_dtype) && y && scale && out && total >= 0, "branch_sum: bad arguments");
+  if (total == 0) return 0;
+  BranchSumArgs a;
+  for (int i = 0; i < kMostBranches; ++i) {
+    a.y[i] = i < count ? y[i] : nullptr;
+    a.scale[i] = i < count ? scale[i] : 0.0f;
+    NNIS_REQUIRE(i >= count || a.y[i], "branch_sum: branch %d has no input", i);
+  }
+  a.count = count; a.y_dtype = y_dtype; a.out = out; a.out_dtype = out_dtype; a.total = (size_t)total;
+  size_t blocks = ((size_t)total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(branch_sum_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("branch_sum");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// Logits times a constant, in place (32-bit rows)
+// -----------------------------------------------------------------------------
+__global__ void scale_rows_kernel(float* __restrict__ x, float factor, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) x[i] *= factor;
+}
+
+extern "C" int nnis_scale_rows(float* x, float factor, long long total, void* stream) {
+  NNIS_REQUIRE(x && total >= 0, "scale_rows: bad arguments");
+  if (total == 0) return 0;
+  size_t blocks = ((size_t)total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, x, factor, (size_t)total);
+  NNIS_LAUNCH_CHECK("scale_rows");
+  return 0;
+}

@@ -135,6 +135,65 @@ __global__ __launch_bounds__(256) void rms_post_step4_kernel(float* x, const T* 
 }
 
 // -----------------------------------------------------------------------------
+// Between two sublayers of a layer that norms both ways with RMS norms: the way out of the one, the sum into the
+// 32-bit stream and the way into the next in one kernel,
+//   x[row] += y / sqrt(mean(y^2) + eps) * w_out;   h[row] = x / sqrt(mean(x^2) + eps) * w_in
+// (y may stand for y + keep[row] * h_in[row], as in rms_post_step).  A block a row; a thread keeps up to kPostKeep
+// values of the row in registers between the three passes and reads what lies beyond again.
+// -----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rms_between_kernel(float* x, const void* __restrict__ y, int y_dtype, const void* __restrict__ w_out,
+                                                          const void* __restrict__ w_in, int w_dtype, float eps, void* h, int h_dtype,
+                                                          int width, const float* __restrict__ keep, const void* __restrict__ h_in,
+                                                          int h_in_dtype) {
+  __shared__ float scratch[16];
+  __shared__ float scratch2[16];
+  const size_t base = (size_t)blockIdx.x * width;
+  const float share = keep ? keep[blockIdx.x] : 0.0f;
+  float vs[kPostKeep];
+  float ss = 0.0f;
+  auto value = [&](int c) {
+    float v = load_as_f32(y, y_dtype, base + c);
+    if (keep) v = fmaf(share, load_as_f32(h_in, h_in_dtype, base + c), v);
+    return v;
+  };
+#pragma unroll
+  for (int i = 0; i < kPostKeep; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    vs[i] = c < width ? value(c) : 0.0f;
+    ss = fmaf(vs[i], vs[i], ss);
+  }
+  for (int c = threadIdx.x + kPostKeep * blockDim.x; c < width; c += blockDim.x) {
+    const float v = value(c);
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  float ss2 = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kPostKeep; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    if (c < width) {
+      vs[i] = x[base + c] + vs[i] * inv * load_as_f32(w_out, w_dtype, c);
+      x[base + c] = vs[i];
+      ss2 = fmaf(vs[i], vs[i], ss2);
+    }
+  }
+  for (int c = threadIdx.x + kPostKeep * blockDim.x; c < width; c += blockDim.x) {
+    const float sum = x[base + c] + value(c) * inv * load_as_f32(w_out, w_dtype, c);
+    x[base + c] = sum;
+    ss2 = fmaf(sum, sum, ss2);
+  }
+  if (h == nullptr) return;
+  const float inv2 = 1.0f / sqrtf(block_sum(ss2, scratch2) / (float)width + eps);
+#pragma unroll
+  for (int i = 0; i < kPostKeep; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    if (c < width) store_from_f32(h, h_dtype, base + c, vs[i] * inv2 * load_as_f32(w_in, w_dtype, c));
+  }
+  for (int c = threadIdx.x + kPostKeep * blockDim.x; c < width; c += blockDim.x)
+    store_from_f32(h, h_dtype, base + c, x[base + c] * inv2 * load_as_f32(w_in, w_dtype, c));
+}
+
+// -----------------------------------------------------------------------------
 // PolyNorm: out = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e, powers element by element, each root mean
 // square over the row with eps inside the root; coef = (a, b, c, e) in device memory.
 // -----------------------------------------------------------------------------
@@ -225,8 +284,11 @@ __global__ __launch_bounds__(256) void poly_norm4_kernel(const T* __restrict__ z
 constexpr int kRouteMost = 16;  // outputs a lane holds: n <= 64 * kRouteMost
 
 // one row by one wave; `logits`: the row's n logits (global memory or LDS)
+// group_count > 1: the outputs form that many equal groups of neighbours; a group's mark is its largest corrected
+// score, and only outputs of the group_keep groups with the largest marks (the lower group on a tie) can be chosen.
 __device__ __forceinline__ void route_row(const float* logits, const float* __restrict__ correction, int row, int n, int experts, int top,
-                                          float* __restrict__ gates, float* __restrict__ keep, int lane) {
+                                          float* __restrict__ gates, float* __restrict__ keep, int lane, int group_count = 1,
+                                          int group_keep = 1) {
   float s[kRouteMost], choice[kRouteMost];
   float top_logit = -INFINITY;
 #pragma unroll
@@ -250,6 +312,42 @@ __device__ __forceinline__ void route_row(const float* logits, const float* __re
     s[i] *= inv;
     choice[i] = e < n ? s[i] + (correction ? correction[e] : 0.0f) : -INFINITY;
   }
+  if (group_count > 1 && group_keep < group_count) {
+    // lane g holds group g's mark (up to 64 groups); the kept groups are found one at a time
+    const int size = n / group_count;
+    float mark = -INFINITY;
+    for (int g = 0; g < group_count; ++g) {
+      float best = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < kRouteMost; ++i) {
+        const int e = i * kWave + lane;
+        if (e < n && e / size == g) best = fmaxf(best, choice[i]);
+      }
+      best = wave_max(best);
+      if (lane == g) mark = best;
+    }
+    unsigned long long allowed = 0ull;
+    for (int round = 0; round < group_keep; ++round) {
+      float best = lane < group_count && !(allowed >> lane & 1ull) ? mark : -INFINITY;
+      int best_g = lane < group_count && !(allowed >> lane & 1ull) ? lane : 0x7fffffff;
+#pragma unroll
+      for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+        const float other = __shfl_xor(best, offset, kWave);
+        const int other_g = __shfl_xor(best_g, offset, kWave);
+        if (other_g != 0x7fffffff && (best_g == 0x7fffffff || other > best || (other == best && other_g < best_g))) {
+          best = other;
+          best_g = other_g;
+        }
+      }
+      if (best_g == 0x7fffffff) break;
+      allowed |= 1ull << best_g;
+    }
+#pragma unroll
+    for (int i = 0; i < kRouteMost; ++i) {
+      const int e = i * kWave + lane;
+      if (e < n && !(allowed >> (e / size) & 1ull)) choice[i] = -INFINITY;
+    }
+  }
   float kept = 0.0f;
   for (int round = 0; round < top; ++round) {
     float best = -INFINITY;
@@ -257,7 +355,7 @@ __device__ __forceinline__ void route_row(const float* logits, const float* __re
 #pragma unroll
     for (int i = 0; i < kRouteMost; ++i) {
       const int e = i * kWave + lane;
-      if (!(chosen >> i & 1u) && e < n && (choice[i] > best || (choice[i] == best && e < best_e))) {
+      if (!(chosen >> i & 1u) && e < n && choice[i] > -INFINITY && (choice[i] > best || (choice[i] == best && e < best_e))) {
         best = choice[i];
         best_e = e;
       }
@@ -291,10 +389,10 @@ __device__ __forceinline__ void route_row(const float* logits, const float* __re
 
 __global__ __launch_bounds__(256) void route_top_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int rows,
                                                         int n, int experts, int top, float* __restrict__ gates,
-                                                        float* __restrict__ keep) {
+                                                        float* __restrict__ keep, int group_count, int group_keep) {
   const int row = blockIdx.x * 4 + threadIdx.x / kWave;
   if (row >= rows) return;
-  route_row(logits + (size_t)row * n, correction, row, n, experts, top, gates, keep, threadIdx.x % kWave);
+  route_row(logits + (size_t)row * n, correction, row, n, experts, top, gates, keep, threadIdx.x % kWave, group_count, group_keep);
 }
 
 // the dot products of R rows with every output's weights, into `out` [R][n] (LDS or global memory with a row stride
@@ -338,7 +436,8 @@ __device__ __forceinline__ void router_dots(const float* xs, const float* __rest
 template <int R>
 __global__ __launch_bounds__(256) void route_kernel(const void* __restrict__ x, int x_dtype, const float* __restrict__ w,
                                                     const float* __restrict__ correction, int rows, int n, int width, int experts,
-                                                    int top, float* __restrict__ gates, float* __restrict__ keep) {
+                                                    int top, float* __restrict__ gates, float* __restrict__ keep, int group_count,
+                                                    int group_keep) {
   extern __shared__ __attribute__((aligned(16))) float lds[];  // [R][width] rows, then [R][n] logits
   float* xs = lds;
   float* lg = lds + (size_t)R * width;
@@ -351,7 +450,8 @@ __global__ __launch_bounds__(256) void route_kernel(const void* __restrict__ x, 
   router_dots<R>(xs, w, lg, n, width);
   __syncthreads();
   const int wave = threadIdx.x / kWave;
-  if (wave < R && row0 + wave < rows) route_row(lg + wave * n, correction, row0 + wave, n, experts, top, gates, keep, threadIdx.x % kWave);
+  if (wave < R && row0 + wave < rows)
+    route_row(lg + wave * n, correction, row0 + wave, n, experts, top, gates, keep, threadIdx.x % kWave, group_count, group_keep);
 }
 
 // the logits alone, to global memory [rows, n]
@@ -396,6 +496,48 @@ __global__ void routed_act_kernel(const void* __restrict__ z, int z_dtype, const
   const float g = gates[row * experts + e];
   const float v = fmaxf(load_as_f32(z, z_dtype, i), 0.0f);
   store_from_f32(out, out_dtype, i, g == 0.0f ? 0.0f : g * v * v);
+}
+
+// The gated form: z [rows, experts * 2 * ff], an expert's gate columns then its up columns;
+// out[row, e * ff + c] = gates[row, e] * silu(z[row, e * 2 ff + c]) * z[row, e * 2 ff + ff + c]
+__global__ void routed_gated_kernel(const void* __restrict__ z, int z_dtype, const float* __restrict__ gates, void* __restrict__ out,
+                                    int out_dtype, int experts, int ff, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t per_row = (size_t)experts * ff;
+  const size_t row = i / per_row;
+  const int e = (int)((i % per_row) / ff), c = (int)(i % ff);
+  const float g = gates[row * experts + e];
+  float v = 0.0f;
+  if (g != 0.0f) {
+    const size_t at = (row * experts + e) * 2 * (size_t)ff + c;
+    const float a = load_as_f32(z, z_dtype, at), u = load_as_f32(z, z_dtype, at + ff);
+    v = g * (a * sigmoid_f(a) * u);
+  }
+  store_from_f32(out, out_dtype, i, v);
+}
+
+// the gated form, eight bfloat16 values a thread (ff a multiple of 8); the gating itself rounds to bfloat16 before the score weighs it
+__global__ void routed_gated_bf16x8_kernel(const bf16_t* __restrict__ z, const float* __restrict__ gates, bf16_t* __restrict__ out,
+                                           int experts, int ff8, size_t total8) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  const size_t per_row = (size_t)experts * ff8;
+  const size_t row = i / per_row;
+  const int e = (int)((i % per_row) / ff8), c8 = (int)(i % ff8);
+  const float g = gates[row * experts + e];
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+  bf16x8_t o = {};
+  if (g != 0.0f) {
+    const bf16_t* at = z + ((row * experts + e) * 2 * (size_t)ff8 + c8) * 8;
+    const bf16x8_t a = *(const bf16x8_t*)at, u = *(const bf16x8_t*)(at + (size_t)ff8 * 8);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float av = (float)a[k];
+      o[k] = (__bf16)(g * (av * sigmoid_f(av) * (float)u[k]));
+    }
+  }
+  *(bf16x8_t*)(out + i * 8) = o;
 }
 
 // the same, eight bfloat16 values a thread (ff a multiple of 8)
@@ -688,6 +830,19 @@ extern "C" int nnis_rms_post_step(float* x, const void* y, int y_dtype, const vo
   return 0;
 }
 
+extern "C" int nnis_rms_between(float* x, const void* y, int y_dtype, const void* w_out, const void* w_in, int w_dtype, float eps, void* h,
+                                int h_dtype, int rows, int width, const float* keep, const void* h_in, int h_in_dtype, void* stream) {
+  NNIS_REQUIRE(x && y && w_out && width > 0 && eps > 0.0f, "rms_between: missing operand");
+  NNIS_REQUIRE((h == nullptr) == (w_in == nullptr), "rms_between: the rows out come with the next norm's weight");
+  NNIS_REQUIRE((keep == nullptr) == (h_in == nullptr) && (h_in == nullptr || nnis_dtype_ok(h_in_dtype)), "rms_between: a share of rows needs both");
+  NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(w_dtype) && (h == nullptr || nnis_dtype_ok(h_dtype)), "rms_between: unknown dtype");
+  if (rows <= 0) return 0;
+  hipLaunchKernelGGL(rms_between_kernel, dim3(rows), dim3(width >= 1024 ? 256 : (width >= 256 ? 128 : 64)), 0, (hipStream_t)stream, x, y,
+                     y_dtype, w_out, w_in, w_dtype, eps, h, h_dtype, width, keep, h_in, h_in_dtype);
+  NNIS_LAUNCH_CHECK("rms_between");
+  return 0;
+}
+
 extern "C" int nnis_poly_norm(const void* z, int z_dtype, const float* coef, float eps, void* out, int out_dtype, int rows, int width,
                               void* stream) {
   NNIS_REQUIRE(z && coef && out && width > 0, "poly_norm: missing operand");
@@ -730,8 +885,10 @@ extern "C" int nnis_router_logits(const void* x, int x_dtype, const float* w, fl
 }
 
 extern "C" int nnis_route(const void* x, int x_dtype, const float* w, const float* correction, int rows, int n, int width, int experts, int top,
-                          float* gates, float* keep, void* stream) {
+                          float* gates, float* keep, int group_count, int group_keep, void* stream) {
   NNIS_REQUIRE(x && w && gates && keep && n > 0 && width > 0, "route: missing operand");
+  NNIS_REQUIRE(group_count >= 1 && group_count <= kWave && n % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
+               "route: %d outputs in %d groups (up to %d, equal ones) of which %d are kept", n, group_count, kWave, group_keep);
   NNIS_REQUIRE(nnis_dtype_ok(x_dtype), "route: unknown dtype");
   NNIS_REQUIRE(n <= kWave * kRouteMost && width <= 8192, "route: up to %d outputs of rows of up to 8192 channels, got %d and %d", kWave * kRouteMost,
                n, width);
@@ -743,34 +900,53 @@ extern "C" int nnis_route(const void* x, int x_dtype, const float* w, const floa
   const dim3 grid((rows + together - 1) / together);
   hipStream_t s = (hipStream_t)stream;
   if (together == 4) {
-    hipLaunchKernelGGL((route_kernel<4>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep);
+    hipLaunchKernelGGL((route_kernel<4>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep,
+                       group_count, group_keep);
   } else if (together == 2) {
-    hipLaunchKernelGGL((route_kernel<2>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep);
+    hipLaunchKernelGGL((route_kernel<2>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep,
+                       group_count, group_keep);
   } else {
-    hipLaunchKernelGGL((route_kernel<1>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep);
+    hipLaunchKernelGGL((route_kernel<1>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep,
+                       group_count, group_keep);
   }
   NNIS_LAUNCH_CHECK("route");
   return 0;
 }
 
 extern "C" int nnis_route_top(const float* logits, const float* correction, int rows, int n, int experts, int top, float* gates,
-                              float* keep, void* stream) {
+                              float* keep, int group_count, int group_keep, void* stream) {
   NNIS_REQUIRE(logits && gates && keep, "route_top: missing operand");
+  NNIS_REQUIRE(group_count >= 1 && group_count <= kWave && n % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
+               "route_top: %d outputs in %d groups (up to %d, equal ones) of which %d are kept", n, group_count, kWave, group_keep);
   NNIS_REQUIRE(n > 0 && n <= kWave * kRouteMost, "route_top: 1 to %d router outputs, got %d", kWave * kRouteMost, n);
   NNIS_REQUIRE(experts >= 0 && experts <= n && top > 0 && top <= n, "route_top: %d experts and the %d largest of %d outputs", experts, top, n);
   if (rows <= 0) return 0;
   hipLaunchKernelGGL(route_top_kernel, dim3((rows + 3) / 4), dim3(256), 0, (hipStream_t)stream, logits, correction, rows, n, experts, top,
-                     gates, keep);
+                     gates, keep, group_count, group_keep);
   NNIS_LAUNCH_CHECK("route_top");
   return 0;
 }
 
+// form 0: z [rows, experts * ff], out = score * relu(z)^2; form 1: z [rows, experts * 2 * ff] (gate columns, then up
+// columns, expert by expert), out = score * silu(gate) * up
 extern "C" int nnis_routed_act(const void* z, int z_dtype, const float* gates, void* out, int out_dtype, int rows, int experts, int ff,
-                               void* stream) {
+                               int form, void* stream) {
   NNIS_REQUIRE(z && gates && out && experts > 0 && ff > 0, "routed_act: missing operand");
   NNIS_REQUIRE(nnis_dtype_ok(z_dtype) && nnis_dtype_ok(out_dtype), "routed_act: unknown dtype");
+  NNIS_REQUIRE(form == 0 || form == 1, "routed_act: unknown form %d", form);
   if (rows <= 0) return 0;
   const size_t total = (size_t)rows * experts * ff;
+  if (form == 1) {
+    if (z_dtype == NNIS_BF16 && out_dtype == NNIS_BF16 && ff % 8 == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0) {
+      hipLaunchKernelGGL(routed_gated_bf16x8_kernel, dim3(blocks_for(total / 8, 256)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)z,
+                         gates, (bf16_t*)out, experts, ff / 8, total / 8);
+    } else {
+      hipLaunchKernelGGL(routed_gated_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, (hipStream_t)stream, z, z_dtype, gates, out,
+                         out_dtype, experts, ff, total);
+    }
+    NNIS_LAUNCH_CHECK("routed_act");
+    return 0;
+  }
   if (z_dtype == NNIS_BF16 && out_dtype == NNIS_BF16 && ff % 8 == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0) {
     hipLaunchKernelGGL(routed_act_bf16x8_kernel, dim3(blocks_for(total / 8, 256)), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)z, gates,
                        (bf16_t*)out, experts, ff / 8, total / 8);

@@ -32,6 +32,10 @@ _CORE_SIGNATURES = {
                            _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
     "nnis_rope_kv_write_wide": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT,
                                 _VOID, _INT, _INT, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID],
+    "nnis_rope_kv_write_shared": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT,
+                                  _VOID, _INT, _INT, _INT, _INT, _INT, _INT, _VOID, _INT, _INT, _VOID],
+    "nnis_branch_sum": [_VOID, _VOID, _INT, _INT, _I64, _VOID, _INT, _VOID],
+    "nnis_scale_rows": [_VOID, _FLT, _I64, _VOID],
     "nnis_silu_mul": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_embed_pair": [_VOID, _VOID, _VOID, _INT, _VOID, _INT, _INT, _VOID, _INT, _INT, _I64, _I64, _VOID, _VOID, _INT, _INT, _VOID],
     "nnis_stream_step": [_VOID, _INT, _INT, _INT, _VOID, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _FLT, _VOID, _INT,
@@ -97,6 +101,10 @@ _RECURRENT_SIGNATURES = {
                             _VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID],
     "nnis_gla_scan": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _FLT, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT,
                       _VOID, _INT, _INT, _VOID, _VOID, _VOID],
+    "nnis_gla_scan_turned": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _VOID, _FLT, _VOID,
+                             _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT, _INT, _VOID, _VOID, _VOID],
+    "nnis_gated_delta": [_VOID, _INT, _INT, _VOID, _VOID, _VOID, _FLT, _FLT, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID,
+                         _VOID],
     "nnis_gla_decays": [_VOID, _VOID, _INT, _INT, _FLT, _VOID],
     "nnis_head_norm_gate": [_VOID, _VOID, _INT, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _FLT, _VOID],
     "nnis_min_gru": [_VOID, _INT, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT, _INT, _VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID],
@@ -105,11 +113,12 @@ _RECURRENT_SIGNATURES = {
 _SUBLAYER_SIGNATURES = {
     "nnis_cast_rows": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _VOID],
     "nnis_rms_post_step": [_VOID, _VOID, _INT, _VOID, _INT, _FLT, _FLT, _VOID, _INT, _INT, _INT, _VOID, _VOID, _INT, _VOID],
-    "nnis_route": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID],
+    "nnis_rms_between": [_VOID, _VOID, _INT, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _VOID, _VOID, _INT, _VOID],
+    "nnis_route": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _VOID, _INT, _INT, _VOID],
     "nnis_poly_norm": [_VOID, _INT, _VOID, _FLT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_router_logits": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _VOID],
-    "nnis_route_top": [_VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID],
-    "nnis_routed_act": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_route_top": [_VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _INT, _INT, _VOID],
+    "nnis_routed_act": [_VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
     "nnis_rows_axpy": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _VOID],
     "nnis_sigmoid_gate": [_VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_head_norm_write": [_VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID, _VOID, _INT, _FLT, _VOID, _VOID, _INT, _INT, _INT,
@@ -123,6 +132,8 @@ _LATENT_SIGNATURES = {
                             _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID],
     "nnis_latent_rotate_q": [_VOID, _INT, _INT, _INT, _INT, _INT, _INT, _VOID, _VOID, _INT, _VOID, _VOID],
     "nnis_head_scale": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_head_scale_of": [_VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_heads_linear": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
 }
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -350,8 +361,11 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
 def rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                   rot_dim: int, tok_slot: torch.Tensor, tok_pos: torch.Tensor, k_pages: Optional[torch.Tensor],
                   v_pages: Optional[torch.Tensor], block_table: Optional[torch.Tensor], heads: int, kv_heads: int,
-                  head_dim: int, value_dim: Optional[int] = None, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Rotates queries and keys by their positions and writes keys and values
+                  head_dim: int, value_dim: Optional[int] = None, bias: Optional[torch.Tensor] = None,
+                  values_from_keys: bool = False) -> torch.Tensor:
+    """``values_from_keys``: the rows hold queries and keys only, and a head's
+    value is its key as projected, before the rotation.
+    Rotates queries and keys by their positions and writes keys and values
     into the pages of each token's slot.  ``k_pages`` and ``v_pages`` are
     ``[pages, *k_page_shape(kv_heads, head_dim)]`` and ``[pages,
     *v_page_shape(kv_heads, value_dim)]`` (``cache/layout.py``); both ``None``
@@ -361,7 +375,9 @@ def rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, cos: Optional[torch.Te
     _dev(qkv, "qkv"), _dev(q_out, "q_out"), _dev(tok_slot, "tok_slot"), _dev(tok_pos, "tok_pos")
     tokens = qkv.shape[0]
     value_dim = value_dim or head_dim
-    if qkv.shape[1] != (heads + kv_heads) * head_dim + kv_heads * value_dim or q_out.shape != (tokens, heads * head_dim):
+    if values_from_keys and value_dim != head_dim:
+        raise KernelError(f"rope_kv_write: values that are the keys have their size ({head_dim}), not {value_dim}")
+    if qkv.shape[1] != (heads + kv_heads) * head_dim + (0 if values_from_keys else kv_heads * value_dim) or q_out.shape != (tokens, heads * head_dim):
         raise KernelError(f"rope_kv_write: qkv {tuple(qkv.shape)} / q_out {tuple(q_out.shape)} do not fit "
                           f"{heads}+{kv_heads} heads of {head_dim} and {kv_heads} of {value_dim}")
     if bias is not None:
@@ -387,11 +403,11 @@ def rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, cos: Optional[torch.Te
         max_pages = block_table.shape[1]
         cache_code = _code(k_pages)
     lib = core()
-    _check(lib, lib.nnis_rope_kv_write_wide(qkv.data_ptr(), _code(qkv), q_out.data_ptr(), _code(q_out), _ptr(cos), _ptr(sin),
-                                            table_positions, rot_dim, tok_slot.data_ptr(), tok_pos.data_ptr(),
-                                            _ptr(k_pages), _ptr(v_pages), cache_code, _ptr(block_table), max_pages, tokens,
-                                            heads, kv_heads, head_dim, value_dim, _ptr(bias),
-                                            _code(bias) if bias is not None else 0, _stream()))
+    _check(lib, lib.nnis_rope_kv_write_shared(qkv.data_ptr(), _code(qkv), q_out.data_ptr(), _code(q_out), _ptr(cos), _ptr(sin),
+                                              table_positions, rot_dim, tok_slot.data_ptr(), tok_pos.data_ptr(),
+                                              _ptr(k_pages), _ptr(v_pages), cache_code, _ptr(block_table), max_pages, tokens,
+                                              heads, kv_heads, head_dim, value_dim, _ptr(bias),
+                                              _code(bias) if bias is not None else 0, 1 if values_from_keys else 0, _stream()))
     return q_out
 
 
@@ -1627,12 +1643,16 @@ def gla_decays(logits: torch.Tensor, bias: torch.Tensor, tau: float) -> torch.Te
     return logits
 
 
-def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_logs: torch.Tensor, scale: float,
-             state: torch.Tensor, ctx, heads: int, out: torch.Tensor) -> torch.Tensor:
+def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_logs: Optional[torch.Tensor], scale: float,
+             state: torch.Tensor, ctx, heads: int, out: torch.Tensor, head_decay: Optional[torch.Tensor] = None,
+             rotation=None) -> torch.Tensor:
     """Gated linear attention over each sequence's tokens, from and into ``state`` (float32 [slots, heads, key
     channels, value channels]): alpha = exp(decay_logs); S <- diag(alpha) S + k v^T; out = S^T (q * scale), raw,
     float32 [tokens, heads * value channels].  q, k [tokens, heads * key channels] and v are views whose rows may be
-    further apart; ``decay_logs`` float32 [tokens, heads * key channels] (``gla_decays``)."""
+    further apart; ``decay_logs`` float32 [tokens, heads * key channels] (``gla_decays``).  Without ``decay_logs``:
+    ``head_decay`` float32 [2, heads], one fixed decay a head and its logarithm (retention).  ``rotation``: (cos, sin,
+    rot_dim): the first rot_dim channels of every head of q and k are turned by the token's position while the kernel
+    stages them, channel i with channel i + rot_dim / 2, in 32-bit (tables float32 [positions, rot_dim / 2])."""
     decay_logits = decay_logs
     tokens = q.shape[0]
     key_dim, value_dim = q.shape[1] // heads, v.shape[1] // heads
@@ -1641,9 +1661,25 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_logs: torc
             raise KernelError(f"gla_scan: {what} must be [tokens, channels] on the GPU with adjacent columns, of one type")
     if k.shape[1] != heads * key_dim or q.shape[1] != heads * key_dim or v.shape[1] != heads * value_dim:
         raise KernelError(f"gla_scan: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not fit {heads} heads")
-    _dev(decay_logits, "decay_logits"), _dev(state, "state"), _dev(out, "out")
-    if decay_logits.dtype != torch.float32 or tuple(decay_logits.shape) != (tokens, heads * key_dim):
-        raise KernelError("gla_scan: decay_logits must be float32 [tokens, heads * key channels]")
+    _dev(state, "state"), _dev(out, "out")
+    if (decay_logits is None) == (head_decay is None):
+        raise KernelError("gla_scan: decays a token and channel, or one a head")
+    if decay_logits is not None:
+        _dev(decay_logits, "decay_logits")
+        if decay_logits.dtype != torch.float32 or tuple(decay_logits.shape) != (tokens, heads * key_dim):
+            raise KernelError("gla_scan: decay_logits must be float32 [tokens, heads * key channels]")
+    else:
+        _dev(head_decay, "head_decay")
+        if head_decay.dtype != torch.float32 or tuple(head_decay.shape) != (2, heads) or not head_decay.is_contiguous():
+            raise KernelError(f"gla_scan: head_decay must be float32 [2, {heads}], got {tuple(head_decay.shape)}")
+    cos = sin = None
+    rot_dim = 0
+    if rotation is not None:
+        cos, sin, rot_dim = rotation
+        _dev(cos, "cos"), _dev(sin, "sin")
+        if (cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.dim() != 2
+                or cos.shape[1] != rot_dim // 2 or rot_dim % 2 or rot_dim > key_dim or ctx.tok_pos.numel() < tokens):
+            raise KernelError(f"gla_scan: tables {tuple(cos.shape)} do not fit a rotation of {rot_dim} channels in heads of {key_dim}")
     if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, key_dim, value_dim):
         raise KernelError(f"gla_scan: state must be float32 [slots, {heads}, {key_dim}, {value_dim}], got {tuple(state.shape)}")
     if out.dtype != torch.float32 or tuple(out.shape) != (tokens, heads * value_dim):
@@ -1656,28 +1692,90 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_logs: torc
         carried = torch.empty(ctx.batch * pieces * heads * key_dim * value_dim, dtype=torch.float32, device=out.device)
         decayed = torch.empty(ctx.batch * pieces * heads * key_dim, dtype=torch.float32, device=out.device)
     lib = recurrent()
-    _check(lib, lib.nnis_gla_scan(q.data_ptr(), k.data_ptr(), v.data_ptr(), _code(q), stride(q), stride(k), stride(v),
-                                  decay_logits.data_ptr(), float(scale), state.data_ptr(), ctx.seq_slot.data_ptr(),
-                                  ctx.seq_start.data_ptr(), ctx.batch, heads, key_dim, value_dim, out.data_ptr(), piece, pieces,
-                                  _ptr(carried), _ptr(decayed), _stream()))
+    _check(lib, lib.nnis_gla_scan_turned(q.data_ptr(), k.data_ptr(), v.data_ptr(), _code(q), stride(q), stride(k), stride(v),
+                                         _ptr(decay_logits), _ptr(head_decay), _ptr(cos), _ptr(sin), rot_dim,
+                                         cos.shape[0] if cos is not None else 0, ctx.tok_pos.data_ptr(), float(scale),
+                                         state.data_ptr(), ctx.seq_slot.data_ptr(), ctx.seq_start.data_ptr(), ctx.batch, heads,
+                                         key_dim, value_dim, out.data_ptr(), piece, pieces, _ptr(carried), _ptr(decayed), _stream()))
     return out
 
 
-def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, out: torch.Tensor) -> torch.Tensor:
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], eps: float, heads: int, out: torch.Tensor) -> torch.Tensor:
     """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight * silu(gate[t, h, :]); ``o`` float32
-    [tokens, heads * dim], ``gate`` a view of that shape whose rows may be further apart, ``weight`` [dim]."""
-    _dev(o, "o"), _dev(weight, "weight"), _dev(out, "out")
+    [tokens, heads * dim], ``gate`` a view of that shape whose rows may be further apart, ``weight`` [dim] or None
+    (a norm without a weight)."""
+    _dev(o, "o"), _dev(out, "out")
     tokens = o.shape[0]
     dim = o.shape[1] // heads
-    if o.dtype != torch.float32 or o.shape[1] != heads * dim or weight.numel() != dim or tuple(out.shape) != tuple(o.shape):
-        raise KernelError(f"head_norm_gate: o {tuple(o.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)} do not fit {heads} heads")
+    if weight is not None:
+        _dev(weight, "weight")
+    if o.dtype != torch.float32 or o.shape[1] != heads * dim or (weight is not None and weight.numel() != dim) or tuple(out.shape) != tuple(o.shape):
+        raise KernelError(f"head_norm_gate: o {tuple(o.shape)}, weight, out {tuple(out.shape)} do not fit {heads} heads")
     if not gate.is_cuda or tuple(gate.shape) != tuple(o.shape) or gate.stride(1) != 1:
         raise KernelError("head_norm_gate: the gate must be [tokens, heads * dim] on the GPU with adjacent columns")
     lib = recurrent()
     _check(lib, lib.nnis_head_norm_gate(o.data_ptr(), gate.data_ptr(), _code(gate), gate.stride(0) if tokens > 1 else gate.shape[1],
-                                        weight.data_ptr(), _code(weight), out.data_ptr(), _code(out), tokens, heads, dim, float(eps),
-                                        _stream()))
+                                        _ptr(weight), _code(weight) if weight is not None else 0, out.data_ptr(), _code(out), tokens,
+                                        heads, dim, float(eps), _stream()))
     return out
+
+
+def gated_delta(rows: torch.Tensor, ba: torch.Tensor, rate: torch.Tensor, dt_bias: torch.Tensor, q_scale: float, state: torch.Tensor,
+                ctx, heads: int, groups: int, key_dim: int, value_dim: int, out: torch.Tensor, unit_eps: float = 1e-6) -> torch.Tensor:
+    """The gated delta rule over each sequence's tokens, from and into ``state`` (float32 [slots, heads, key channels,
+    value channels]): S <- g S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q, raw, float32 [tokens, heads * value
+    channels].  ``rows`` [tokens, >= 2 * groups * key_dim + heads * value_dim]: q and k of ``groups`` heads, then v; q
+    and k are made unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q also times ``q_scale``.  ``ba`` float32
+    [tokens, 2 * heads]: beta = sigmoid(first half), g = exp(-rate * softplus(second half + dt_bias)); ``rate`` and
+    ``dt_bias`` float32 [heads]."""
+    _dev(rows, "rows"), _dev(ba, "ba"), _dev(rate, "rate"), _dev(dt_bias, "dt_bias"), _dev(state, "state"), _dev(out, "out")
+    tokens = rows.shape[0]
+    if rows.dim() != 2 or rows.stride(1) != 1 or rows.shape[1] < 2 * groups * key_dim + heads * value_dim:
+        raise KernelError(f"gated_delta: rows {tuple(rows.shape)} do not hold {groups} query/key heads of {key_dim} and {heads} values of {value_dim}")
+    if ba.dtype != torch.float32 or tuple(ba.shape) != (tokens, 2 * heads) or not ba.is_contiguous():
+        raise KernelError(f"gated_delta: ba must be float32 [tokens, {2 * heads}], got {tuple(ba.shape)}")
+    for t, what in ((rate, "rate"), (dt_bias, "dt_bias")):
+        if t.dtype != torch.float32 or t.numel() != heads:
+            raise KernelError(f"gated_delta: {what} must be float32 [{heads}]")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, key_dim, value_dim):
+        raise KernelError(f"gated_delta: state must be float32 [slots, {heads}, {key_dim}, {value_dim}], got {tuple(state.shape)}")
+    if out.dtype != torch.float32 or tuple(out.shape) != (tokens, heads * value_dim):
+        raise KernelError("gated_delta: out must be float32 [tokens, heads * value channels]")
+    _step_arrays(ctx, "gated_delta")
+    lib = recurrent()
+    _check(lib, lib.nnis_gated_delta(rows.data_ptr(), _code(rows), rows.stride(0) if tokens > 1 else rows.shape[1], ba.data_ptr(),
+                                     rate.data_ptr(), dt_bias.data_ptr(), float(q_scale), float(unit_eps), state.data_ptr(),
+                                     ctx.seq_slot.data_ptr(), ctx.seq_start.data_ptr(), ctx.batch, heads, groups, key_dim, value_dim,
+                                     out.data_ptr(), _stream()))
+    return out
+
+
+def branch_sum(branches, scales, out: torch.Tensor) -> torch.Tensor:
+    """out = sum over the branches of scale * y: up to four inputs of one type and of out's shape, the sum in 32-bit."""
+    count = len(branches)
+    if not 1 <= count <= 4 or len(scales) != count:
+        raise KernelError("branch_sum: one to four branches, each with a factor")
+    _dev(out, "out")
+    for y in branches:
+        _dev(y, "branch")
+        if y.shape != out.shape or y.dtype != branches[0].dtype or not y.is_contiguous():
+            raise KernelError("branch_sum: branches must agree with the output in shape and with one another in type")
+    ys = (ctypes.c_void_p * count)(*[y.data_ptr() for y in branches])
+    factors = (ctypes.c_float * count)(*[float(value) for value in scales])
+    lib = core()
+    _check(lib, lib.nnis_branch_sum(ctypes.cast(ys, _VOID), ctypes.cast(factors, _VOID), count, _code(branches[0]), out.numel(),
+                                    out.data_ptr(), _code(out), _stream()))
+    return out
+
+
+def scale_rows(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """x *= factor, in place, on 32-bit rows."""
+    _dev(x, "x")
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError(f"scale_rows: 32-bit rows are needed, got {x.dtype}")
+    lib = core()
+    _check(lib, lib.nnis_scale_rows(x.data_ptr(), float(factor), x.numel(), _stream()))
+    return x
 
 
 # ---------------------------------------------------------------------------
@@ -1830,15 +1928,39 @@ def latent_rotate_q(q: torch.Tensor, heads: int, head_width: int, first: int, ro
     return q
 
 
-def head_scale(o: torch.Tensor, gate: torch.Tensor, heads: int) -> torch.Tensor:
-    """o[t, h, :] *= gate[t, h], in place; ``o`` [tokens, heads * channels], ``gate`` float32 [tokens, heads]."""
+def head_scale(o: torch.Tensor, gate: torch.Tensor, heads: int, logistic: bool = False) -> torch.Tensor:
+    """o[t, h, :] *= gate[t, h], in place; ``o`` [tokens, heads * channels], ``gate`` float32 [tokens, heads].
+    ``logistic``: the gates are logits still, and the factor is sigmoid(gate[t, h])."""
     _dev(o, "o"), _dev(gate, "gate")
     tokens = o.shape[0]
     if o.shape[1] % heads or gate.shape != (tokens, heads) or gate.dtype != torch.float32:
         raise KernelError(f"head_scale: o {tuple(o.shape)} and gate {tuple(gate.shape)} {gate.dtype} do not fit {heads} heads")
     lib = latent()
-    _check(lib, lib.nnis_head_scale(o.data_ptr(), _code(o), gate.data_ptr(), tokens, heads, o.shape[1] // heads, _stream()))
+    if not gate.is_contiguous() or not o.is_contiguous():
+        raise KernelError("head_scale: rows and gates lie one behind the other")
+    _check(lib, lib.nnis_head_scale_of(o.data_ptr(), _code(o), gate.data_ptr(), tokens, heads, o.shape[1] // heads,
+                                       1 if logistic else 0, _stream()))
     return o
+
+
+def heads_linear(x: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.Tensor], heads: int, out: torch.Tensor) -> torch.Tensor:
+    """out[t, h, :] = (weight[h] @ x[t, h, :]) * gate[t, h, :]: a map of its own for every head.  ``x`` [tokens, heads *
+    K], ``weight`` [heads, N, K], ``gate`` float32 [tokens, heads * N] or None, ``out`` [tokens, heads * N]."""
+    _dev(x, "x"), _dev(weight, "weight"), _dev(out, "out")
+    tokens = x.shape[0]
+    if weight.dim() != 3 or weight.shape[0] != heads or not weight.is_contiguous() or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError(f"heads_linear: a weight [heads, N, K] is needed, got {tuple(weight.shape)}")
+    n, k = weight.shape[1], weight.shape[2]
+    if tuple(x.shape) != (tokens, heads * k) or tuple(out.shape) != (tokens, heads * n):
+        raise KernelError(f"heads_linear: x {tuple(x.shape)} and out {tuple(out.shape)} against {heads} maps of {n} x {k}")
+    if gate is not None:
+        _dev(gate, "gate")
+        if gate.dtype != torch.float32 or tuple(gate.shape) != (tokens, heads * n) or not gate.is_contiguous():
+            raise KernelError(f"heads_linear: the gate must be float32 [tokens, {heads * n}], got {tuple(gate.shape)}")
+    lib = latent()
+    _check(lib, lib.nnis_heads_linear(x.data_ptr(), _code(x), weight.data_ptr(), _code(weight), _ptr(gate), out.data_ptr(), _code(out),
+                                      tokens, heads, n, k, _stream()))
+    return out
 
 
 # ---------------------------------------------------------------------------
@@ -1884,6 +2006,33 @@ def rms_post_step(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, offset
     return h
 
 
+def rms_between(x: torch.Tensor, y: torch.Tensor, w_out: torch.Tensor, w_in: Optional[torch.Tensor], eps: float,
+                h: Optional[torch.Tensor] = None, share=None) -> Optional[torch.Tensor]:
+    """Between two sublayers that are normed both ways: x += y / sqrt(mean(y^2) + eps) * w_out, row by row, in place in
+    the 32-bit stream ``x``, and h = x / sqrt(mean(x^2) + eps) * w_in (``h`` and ``w_in`` together, or neither).
+    ``share`` as in ``rms_post_step``.  The two weights have one type."""
+    _dev(x, "x"), _dev(y, "y"), _dev(w_out, "norm weight")
+    if x.dtype != torch.float32 or x.dim() != 2 or y.shape != x.shape or w_out.numel() != x.shape[1] or not y.is_contiguous():
+        raise KernelError(f"rms_between: a float32 stream {tuple(x.shape)} against y {tuple(y.shape)} and a weight of {w_out.numel()}")
+    if (h is None) != (w_in is None):
+        raise KernelError("rms_between: the rows out come with the next norm's weight")
+    if h is not None:
+        _dev(h, "h"), _dev(w_in, "next norm weight")
+        if h.shape != x.shape or w_in.numel() != x.shape[1] or w_in.dtype != w_out.dtype:
+            raise KernelError(f"rms_between: h {tuple(h.shape)} and the next weight against the stream {tuple(x.shape)}")
+    keep = rows_in = None
+    if share is not None:
+        keep, rows_in = share
+        _dev(keep, "keep"), _dev(rows_in, "shared rows")
+        if keep.dtype != torch.float32 or keep.numel() != x.shape[0] or rows_in.shape != x.shape or not rows_in.is_contiguous():
+            raise KernelError(f"rms_between: a float32 share per row and rows {tuple(x.shape)}, got {tuple(keep.shape)} and {tuple(rows_in.shape)}")
+    lib = sublayer()
+    _check(lib, lib.nnis_rms_between(x.data_ptr(), y.data_ptr(), _code(y), w_out.data_ptr(), _ptr(w_in), _code(w_out), float(eps), _ptr(h),
+                                     _code(h) if h is not None else 0, x.shape[0], x.shape[1], _ptr(keep), _ptr(rows_in),
+                                     _code(rows_in) if rows_in is not None else 0, _stream()))
+    return h
+
+
 def poly_norm(z: torch.Tensor, coefficients: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
     """out = a N(z) + b N(z^2) + c N(z^3) + e row by row, N(v) = v / sqrt(mean(v^2) + eps); ``coefficients``: float32
     (a, b, c, e) on the device."""
@@ -1913,8 +2062,18 @@ def router_logits(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> t
     return out
 
 
+def _route_groups(groups, n: int, what: str):
+    """(count, keep) of a router whose outputs form equal groups of neighbours, (1, 1) without."""
+    if groups is None:
+        return 1, 1
+    count, keep = int(groups[0]), int(groups[1])
+    if not (1 <= count <= 64 and n % count == 0 and 1 <= keep <= count):
+        raise KernelError(f"{what}: {n} outputs in {count} equal groups (up to 64) of which {keep} are kept")
+    return count, keep
+
+
 def route_top(logits: torch.Tensor, correction: Optional[torch.Tensor], experts: int, top: int, gates: torch.Tensor,
-              keep: torch.Tensor):
+              keep: torch.Tensor, groups=None):
     """Scores softmax(logits) [rows, n]; the ``top`` largest of score + correction are chosen.  ``gates`` [rows, experts]
     gets the score of every chosen output below ``experts`` and 0 elsewhere; ``keep`` [rows] the summed scores of the
     chosen outputs from ``experts`` on.  All float32."""
@@ -1929,8 +2088,10 @@ def route_top(logits: torch.Tensor, correction: Optional[torch.Tensor], experts:
             raise KernelError(f"route_top: a float32 correction per output ({n}), got {tuple(correction.shape)} {correction.dtype}")
     if not (0 < n <= ROUTE_MOST_OUTPUTS and 0 <= experts <= n and 0 < top <= n):
         raise KernelError(f"route_top: {experts} experts and the {top} largest of {n} outputs (at most {ROUTE_MOST_OUTPUTS})")
+    group_count, group_keep = _route_groups(groups, n, "route_top")
     lib = sublayer()
-    _check(lib, lib.nnis_route_top(logits.data_ptr(), _ptr(correction), rows, n, experts, top, gates.data_ptr(), keep.data_ptr(), _stream()))
+    _check(lib, lib.nnis_route_top(logits.data_ptr(), _ptr(correction), rows, n, experts, top, gates.data_ptr(), keep.data_ptr(),
+                                   group_count, group_keep, _stream()))
     return gates, keep
 
 
@@ -1938,8 +2099,10 @@ ROUTE_FUSED_MOST_CHANNELS = 8192
 
 
 def route(x: torch.Tensor, weight: torch.Tensor, correction: Optional[torch.Tensor], experts: int, top: int, gates: torch.Tensor,
-          keep: torch.Tensor):
-    """``router_logits`` and ``route_top`` in one kernel (rows of up to ``ROUTE_FUSED_MOST_CHANNELS`` channels)."""
+          keep: torch.Tensor, groups=None):
+    """``router_logits`` and ``route_top`` in one kernel (rows of up to ``ROUTE_FUSED_MOST_CHANNELS`` channels).
+    ``groups``: (count, keep): the outputs form ``count`` equal groups of neighbours, a group's mark is its largest
+    corrected score, and only outputs of the ``keep`` groups with the largest marks can be chosen."""
     _dev(x, "x"), _dev(weight, "router weight"), _dev(gates, "gates"), _dev(keep, "keep")
     rows, width = x.shape
     n = weight.shape[0]
@@ -1952,21 +2115,28 @@ def route(x: torch.Tensor, weight: torch.Tensor, correction: Optional[torch.Tens
             raise KernelError(f"route: a float32 correction per output ({n}), got {tuple(correction.shape)} {correction.dtype}")
     if not (0 < n <= ROUTE_MOST_OUTPUTS and 0 <= experts <= n and 0 < top <= n and width <= ROUTE_FUSED_MOST_CHANNELS):
         raise KernelError(f"route: {experts} experts and the {top} largest of {n} outputs (at most {ROUTE_MOST_OUTPUTS}) of rows of {width} channels")
+    group_count, group_keep = _route_groups(groups, n, "route")
     lib = sublayer()
     _check(lib, lib.nnis_route(x.data_ptr(), _code(x), weight.data_ptr(), _ptr(correction), rows, n, width, experts, top, gates.data_ptr(),
-                               keep.data_ptr(), _stream()))
+                               keep.data_ptr(), group_count, group_keep, _stream()))
     return gates, keep
 
 
-def routed_act(z: torch.Tensor, gates: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[row, e * ff + c] = gates[row, e] * relu(z[row, e * ff + c])^2 on the experts' fused up projection."""
+def routed_act(z: torch.Tensor, gates: torch.Tensor, out: torch.Tensor, form: str = "relu_squared") -> torch.Tensor:
+    """On the experts' fused up projection.  ``relu_squared``: out[row, e * ff + c] = gates[row, e] * relu(z[row, e * ff
+    + c])^2.  ``silu_gated``: z [rows, experts * 2 * ff] holds, expert by expert, gate columns then up columns, and
+    out[row, e * ff + c] = gates[row, e] * silu(gate) * up."""
     _dev(z, "z"), _dev(gates, "gates"), _dev(out, "out")
     rows, experts = gates.shape
-    if gates.dtype != torch.float32 or z.dim() != 2 or z.shape[0] != rows or z.shape[1] % max(experts, 1) or out.shape != z.shape:
+    if form not in ("relu_squared", "silu_gated"):
+        raise KernelError(f"routed_act: unknown form {form!r}")
+    per = 2 if form == "silu_gated" else 1
+    if (gates.dtype != torch.float32 or z.dim() != 2 or z.shape[0] != rows or z.shape[1] % max(per * experts, 1)
+            or tuple(out.shape) != (rows, z.shape[1] // per) or not z.is_contiguous() or not out.is_contiguous()):
         raise KernelError(f"routed_act: z {tuple(z.shape)} and out {tuple(out.shape)} against gates {tuple(gates.shape)}")
     lib = sublayer()
     _check(lib, lib.nnis_routed_act(z.data_ptr(), _code(z), gates.data_ptr(), out.data_ptr(), _code(out), rows, experts,
-                                    z.shape[1] // experts, _stream()))
+                                    z.shape[1] // (per * experts), per - 1, _stream()))
     return out
 
 

@@ -13,7 +13,9 @@ a rotation of the first channels of a head only (the position encoding's
 ``rot_dim``); with a window, first tokens that stay visible to every later
 query (``keep_first``); a learned bias by distance added to the scaled score
 (``distance_bias``, ``bias_reach``); a sink in the softmax's denominator
-(``sink``).
+(``sink``); values that are the keys as projected, before their rotation, with
+no projection of their own (``values_from_keys``); a gate per head, sigmoid of
+a projection of the mixer's input, on the head's output (``head_gate``).
 """
 
 from __future__ import annotations
@@ -43,7 +45,8 @@ class CausalSelfAttention(Mixer):
 
     def __init__(self, width, heads, kv_heads, head_dim, q, k, v, o, position=None, window=None, positions=None,
                  value_dim=None, scale=None, softcap=None, q_bias=None, k_bias=None, v_bias=None, o_bias=None,
-                 keep_first=None, distance_bias=None, bias_reach=None, bias_buckets=None, sink=None):
+                 keep_first=None, distance_bias=None, bias_reach=None, bias_buckets=None, sink=None, values_from_keys=False,
+                 head_gate=None):
         """``keep_first``: with a ``window``, keys at positions below it stay
         visible.  ``distance_bias``: the name of a table [buckets, heads]; the
         scaled score of a key n positions back gets row ``distance_bucket(n,
@@ -57,10 +60,14 @@ class CausalSelfAttention(Mixer):
         self.value_dim = self.head_dim if value_dim is None else int(value_dim)
         if self.value_dim <= 0:
             raise InvalidInput(f"value_dim must be positive, got {value_dim}")
+        self.values_from_keys = bool(values_from_keys)
+        if self.values_from_keys and (self.value_dim != self.head_dim or v is not None or v_bias is not None):
+            raise InvalidInput("values that are the keys have the keys' size and no projection of their own")
+        self.gate_name, self.gate = head_gate, None
         self.softcap = 0.0 if not softcap else float(softcap)
         if self.softcap < 0.0:
             raise InvalidInput(f"the cap of the scores must be positive, got {softcap}")
-        if (q_bias is None) != (k_bias is None) or (q_bias is None) != (v_bias is None):
+        if (q_bias is None) != (k_bias is None) or ((q_bias is None) != (v_bias is None) and not values_from_keys):
             raise InvalidInput("the projections of queries, keys and values have biases all three or none")
         self.bias_names = {"q": q_bias, "k": k_bias, "v": v_bias, "o": o_bias}
         self.qkv_bias = None
@@ -96,6 +103,10 @@ class CausalSelfAttention(Mixer):
             TensorSpec(self.names["v"], (v_width, self.width)),
             TensorSpec(self.names["o"], (self.width, o_width)),
         ]
+        if self.values_from_keys:
+            del out[2]
+        if self.gate_name:
+            out.append(TensorSpec(self.gate_name, (self.heads, self.width)))
         for key, size in (("q", q_width), ("k", kv_width), ("v", v_width), ("o", self.width)):
             if self.bias_names[key]:
                 out.append(TensorSpec(self.bias_names[key], (size,)))
@@ -107,10 +118,13 @@ class CausalSelfAttention(Mixer):
 
     def bind(self, weights, rt):
         # one projection for queries, keys and values: rows q heads, k heads, v heads
-        self.qkv = Projection(torch.cat([weights[self.names["q"]], weights[self.names["k"]], weights[self.names["v"]]], dim=0), rt)
+        rows = ("q", "k") if self.values_from_keys else ("q", "k", "v")
+        self.qkv = Projection(torch.cat([weights[self.names[key]] for key in rows], dim=0), rt)
         self.out = Projection(weights[self.names["o"]], rt)
+        if self.gate_name:
+            self.gate = Projection(weights[self.gate_name], rt)
         if self.bias_names["q"]:
-            self.qkv_bias = torch.cat([weights[self.bias_names[key]] for key in ("q", "k", "v")]).contiguous()
+            self.qkv_bias = torch.cat([weights[self.bias_names[key]] for key in rows]).contiguous()
         if self.bias_names["o"]:
             self.output_bias = weights[self.bias_names["o"]].contiguous()
         bias = sink = None
@@ -129,7 +143,7 @@ class CausalSelfAttention(Mixer):
         self.extras = rt.ops.ScoreExtras(self.keep_first, bias, sink)
 
     def weight_bytes(self):
-        return self.qkv.weight_bytes() + self.out.weight_bytes()
+        return self.qkv.weight_bytes() + self.out.weight_bytes() + (self.gate.weight_bytes() if self.gate is not None else 0)
 
     def cache_request(self):
         return KVRequest(self.kv_heads, self.head_dim, self.window, None if self.value_dim == self.head_dim else self.value_dim)
@@ -147,7 +161,7 @@ class CausalSelfAttention(Mixer):
     @property
     def _plain(self) -> bool:
         """The formula without any of the options: what the fused kernels of the projections take."""
-        return self.value_dim == self.head_dim and self.qkv_bias is None
+        return self.value_dim == self.head_dim and self.qkv_bias is None and not self.values_from_keys
 
     def decode_plan(self, batch, longest, rt):
         # (runs of the keys, waves of a block) of a step of single tokens with these sizes
@@ -195,13 +209,20 @@ class CausalSelfAttention(Mixer):
             tables.cos if tables else None, tables.sin if tables else None, tables.rot_dim if tables else 0,
             ctx.tok_slot, ctx.tok_pos,
             view.k_pages if writes else None, view.v_pages if writes else None, view.block_table if writes else None,
-            self.heads, self.kv_heads, self.head_dim, self.value_dim, self.qkv_bias,
+            self.heads, self.kv_heads, self.head_dim, self.value_dim, self.qkv_bias, values_from_keys=self.values_from_keys,
         )
         return q
 
     can_leave_bias = True  # ``forward(..., bias_later=True)`` leaves ``output_bias`` to a consumer that adds it in a kernel of its own
 
     def forward(self, x, ctx, view, rt, into=None, bias_later=False):
+        gate = None
+        if self.gate is not None:
+            # (the gates read the mixer's input as the projections do; their logits stay 32-bit)
+            if hasattr(x, "materialize"):
+                x = x.materialize()
+            gate = self.gate(x, rt, out_dtype=torch.float32)
+            into = None  # the heads are gated before the output projection, which then takes plain rows
         q = self._project_rotate_store(x, ctx, view, rt)
         tokens = q.shape[0]
         attn = rt.empty(tokens, self.heads * self.value_dim)
@@ -219,6 +240,8 @@ class CausalSelfAttention(Mixer):
                                 value_dim=self.value_dim, softcap=self.softcap, extras=self.extras)
         if isinstance(attn, rt.ops.KeyRuns) and not (into.can_take(attn, self.out.weight) and attn.fits(self.out.weight.shape[0])):
             attn = attn.combine()
+        if gate is not None:
+            rt.ops.head_scale(attn, gate, self.heads, logistic=True)
         if into is not None and self.output_bias is None and into.can_take(attn, self.out.weight):
             return into.take(attn, self.out.weight)  # the output projection adds to the stream itself
         y = self.out(attn, rt)

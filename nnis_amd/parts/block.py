@@ -261,11 +261,21 @@ class PrePostNormBlock(Block):
         return part.forward(*args)
 
     @staticmethod
-    def _between(x, y, post, following, rt):
-        """x += post(y) in place; returns following(x)."""
-        if hasattr(post, "triple") and hasattr(following, "triple"):
+    def _rms_pair(post, following) -> bool:
+        """Whether both are plain RMS norms of one eps and one weight type: their step between two sublayers is one kernel."""
+        return (getattr(post, "fusable_rms", False) and getattr(following, "fusable_rms", False) and post.eps == following.eps
+                and post.weight is not None and following.weight is not None and post.weight.dtype == following.weight.dtype)
+
+    @classmethod
+    def _between(cls, x, y, post, following, rt, share=None):
+        """x += post(y) in place; returns following(x).  ``share``: (a factor per row, rows): y stands for y + factor * rows."""
+        if hasattr(post, "triple") and hasattr(following, "triple") and share is None:
             return rt.ops.tanh_norm_step(x, x_out=x, y=y, post=post.triple(), following=following.triple(),
                                          h=rt.empty(x.shape[0], x.shape[1]))
+        if cls._rms_pair(post, following) and y.is_contiguous():
+            return rt.ops.rms_between(x, y, post.weight, following.weight, post.eps, h=rt.empty(x.shape[0], x.shape[1]), share=share)
+        if share is not None:
+            rt.ops.rows_axpy(y, share[1], share[0])
         return following.add_forward(x, post.forward(y, rt), rt)
 
     def forward(self, stream, ctx, view, rt, following=None):
@@ -287,14 +297,20 @@ class PrePostNormBlock(Block):
         after_mixer = self.norm2 if self.feed_forward is not None else following
         y = self._run(self.mixer, (h, ctx, view, rt), x, self.post1, after_mixer, rt)
         post = self.post1
+        share = None
         if self.feed_forward is not None:
             h = y.h if isinstance(y, PreparedRows) else self._between(x, y, self.post1, self.norm2, rt)
-            y = self._run(self.feed_forward, (h, ctx, rt), x, self.post2, following, rt)
+            if getattr(self.feed_forward, "can_leave_share", False) and following is not None and self._rms_pair(self.post2, following):
+                # (a feed-forward that hands a share of its input through leaves that sum to the step's kernel)
+                y = self.feed_forward.forward(h, ctx, rt, share_later=True)
+                y, share = y if isinstance(y, tuple) else (y, None)
+            else:
+                y = self._run(self.feed_forward, (h, ctx, rt), x, self.post2, following, rt)
             post = self.post2
         if isinstance(y, PreparedRows):
             return y
-        if following is not None and hasattr(post, "triple") and hasattr(following, "triple"):
-            return PreparedRows(following, x, self._between(x, y, post, following, rt))
+        if following is not None and ((hasattr(post, "triple") and hasattr(following, "triple")) or self._rms_pair(post, following)):
+            return PreparedRows(following, x, self._between(x, y, post, following, rt, share=share))
         return x, PostNormed(y, post)
 
 

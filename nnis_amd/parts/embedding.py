@@ -77,10 +77,11 @@ class PairHashEmbedding(Part):
 class LinearHead(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size, width, weight, tied_to=None, softcap=None):
-        """``softcap``: logits z leave as softcap * tanh(z / softcap)."""
+    def __init__(self, vocab_size, width, weight, tied_to=None, softcap=None, scale=None):
+        """``softcap``: logits z leave as softcap * tanh(z / softcap).  ``scale``: logits are multiplied by it (before a cap)."""
         self.vocab_size, self.width, self.weight_name, self.tied_to = int(vocab_size), int(width), weight, tied_to
         self.softcap = None if not softcap else float(softcap)
+        self.scale = None if scale is None or float(scale) == 1.0 else float(scale)
         self.projection = None
 
     def tensors(self):
@@ -99,6 +100,8 @@ class LinearHead(Part):
     def forward(self, x, rt):
         """Logits are 32-bit whatever the storage type."""
         logits = self.projection(x, rt, out_dtype=torch.float32)
+        if self.scale is not None:
+            rt.ops.scale_rows(logits, self.scale)
         return logits if self.softcap is None else rt.ops.tanh_cap(logits, self.softcap)
 
 

@@ -100,24 +100,38 @@ class PolyNormFeedForward(FeedForward):
 
 
 class RoutedFeedForward(FeedForward):
-    """A mixture of ``experts`` small feed-forwards, down_e(relu(up_e x)^2), of which a token uses ``top``:
+    """A mixture of ``experts`` small feed-forwards, down_e(relu(up_e x)^2) or (``activation="silu_gated"``)
+    down_e(silu(gate_e x) * up_e x), of which a token uses ``top``:
 
         s = softmax(W_r x) over experts + identity outputs       32-bit
         chosen = the ``top`` largest of s + correction           (the lower index on a tie)
         out = sum over chosen e of s_e * expert_e(x),            expert_e(x) = x for the last ``identity`` outputs
 
     The weights are the scores themselves, not renormalised; ``correction`` (a tensor's name or None) enters the
-    choice only.  The experts' up projections are one product over all experts, gated row by row with the scores
-    (zero for the experts not chosen) before one down projection over all of them."""
+    choice only.  ``groups`` (count, keep): the outputs, identity outputs included, form ``count`` equal groups of
+    neighbours; a group's mark is its largest corrected score, and only outputs of the ``keep`` groups with the largest
+    marks can be chosen.  The experts' up projections are one product over all experts, gated row by row with the
+    scores (zero for the experts not chosen) before one down projection over all of them."""
 
     graph_safe = True
 
-    def __init__(self, width, inner, experts, top, router, up, down, identity=0, correction=None):
-        """``up`` and ``down``: names with ``{}`` in the expert's place."""
+    def __init__(self, width, inner, experts, top, router, up, down, identity=0, correction=None, activation="relu_squared", gate=None,
+                 groups=None):
+        """``up``, ``down`` and ``gate``: names with ``{}`` in the expert's place."""
         self.width, self.inner, self.experts, self.top, self.identity = int(width), int(inner), int(experts), int(top), int(identity or 0)
         if min(self.width, self.inner, self.experts, self.top) <= 0 or self.identity < 0 or self.top > self.experts + self.identity:
             raise InvalidInput(f"a router of {experts} experts and {identity} identity outputs cannot choose {top}")
-        self.names = {"router": router, "up": up, "down": down, "correction": correction}
+        if activation not in ("relu_squared", "silu_gated") or (activation == "silu_gated") != (gate is not None):
+            raise InvalidInput(f"experts are relu_squared, or silu_gated with gate projections; got {activation!r}")
+        self.activation = activation
+        self.groups = None
+        if groups is not None and int(groups[0]) > 1:
+            count, keep = int(groups[0]), int(groups[1])
+            outputs = self.experts + self.identity
+            if outputs % count or not 1 <= keep <= count or self.top > keep * (outputs // count):
+                raise InvalidInput(f"{outputs} router outputs in {count} equal groups of which {keep} are kept cannot choose {top}")
+            self.groups = (count, keep)
+        self.names = {"router": router, "up": up, "down": down, "correction": correction, "gate": gate}
 
     def tensors(self):
         n, outputs = self.names, self.experts + self.identity
@@ -125,6 +139,8 @@ class RoutedFeedForward(FeedForward):
         if n["correction"]:
             out.append(TensorSpec(n["correction"], (outputs,), init="small"))
         for e in range(self.experts):
+            if n["gate"]:
+                out.append(TensorSpec(n["gate"].format(e), (self.inner, self.width)))
             out += [TensorSpec(n["up"].format(e), (self.inner, self.width)), TensorSpec(n["down"].format(e), (self.width, self.inner))]
         return out
 
@@ -137,7 +153,9 @@ class RoutedFeedForward(FeedForward):
         n = self.names
         self.router = weights[n["router"]].float().contiguous()  # its logits are a 32-bit product under either runtime
         self.correction = weights[n["correction"]].float().contiguous() if n["correction"] else None
-        self.up = Projection(torch.cat([weights[n["up"].format(e)] for e in range(self.experts)], dim=0), rt)
+        # one product over all experts: expert by expert its up rows (behind its gate rows, where it has them)
+        rows = [weights[name.format(e)] for e in range(self.experts) for name in ((n["gate"], n["up"]) if n["gate"] else (n["up"],))]
+        self.up = Projection(torch.cat(rows, dim=0), rt)
         self.down = Projection(torch.cat([weights[n["down"].format(e)] for e in range(self.experts)], dim=1), rt)
 
     def weight_bytes(self):
@@ -150,12 +168,12 @@ class RoutedFeedForward(FeedForward):
         tokens = x.shape[0]
         gates, keep = rt.empty(tokens, self.experts, dtype=torch.float32), rt.empty(tokens, dtype=torch.float32)
         if self.width <= rt.ops.ROUTE_FUSED_MOST_CHANNELS:
-            rt.ops.route(x, self.router, self.correction, self.experts, self.top, gates, keep)
+            rt.ops.route(x, self.router, self.correction, self.experts, self.top, gates, keep, groups=self.groups)
         else:
             logits = rt.ops.router_logits(x, self.router, rt.empty(tokens, self.experts + self.identity, dtype=torch.float32))
-            rt.ops.route_top(logits, self.correction, self.experts, self.top, gates, keep)
+            rt.ops.route_top(logits, self.correction, self.experts, self.top, gates, keep, groups=self.groups)
         z = self.up(x, rt)
-        y = self.down(rt.ops.routed_act(z, gates, rt.empty(tokens, self.experts * self.inner)), rt)
+        y = self.down(rt.ops.routed_act(z, gates, rt.empty(tokens, self.experts * self.inner), self.activation), rt)
         if self.identity and share_later:
             return y, (keep, x)
         if self.identity:

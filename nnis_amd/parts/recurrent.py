@@ -1,5 +1,6 @@
 """Mixers that carry a state of fixed size from token to token instead of
-keys and values: the selective scan and gated linear attention.  Their state
+keys and values: the selective scan, gated linear attention, retention, the
+gated delta rule and the minGRU.  Their state
 lives in the cache's per-slot regions (``StateRequest``), in 32-bit, zero when
 a sequence starts; a step reads it at each sequence's first row and leaves it
 behind the last, so a prompt gives the same in one step, in portions or token
@@ -166,6 +167,148 @@ class GatedLinearAttention(Mixer):
         return self.out(gated, rt)
 
 
+class Retention(Mixer):
+    """Linear attention with one fixed decay a head and no softmax or denominator.  With H heads, d key and e value
+    channels a head:
+
+        q = rot(W_q h),  k = rot(W_k h) / sqrt(d),  v = W_v h      rot: the first channels of a head turned by the position
+        S <- decay_h S + k v^T,   o = S^T q                        per head, S [d, e]
+        out = W_o (concat_h(o / rms(o)) * silu(W_g h))
+
+    the norm of a head's o over its e channels without a weight.  The state is that of gated linear attention and so
+    is the kernel, with the decay a constant of the head and the rotation done while it stages queries and keys;
+    rotation, state and norm are 32-bit under either runtime."""
+
+    graph_safe = True
+
+    def __init__(self, width, heads, key_dim, value_dim, decay, eps, q, k, v, g, o, position=None, positions=None):
+        self.width, self.heads, self.key_dim, self.value_dim = int(width), int(heads), int(key_dim), int(value_dim)
+        self.eps = float(eps)
+        self.decay = [float(value) for value in decay]
+        if min(self.heads, self.key_dim, self.value_dim) <= 0 or len(self.decay) != self.heads or not all(0.0 < d <= 1.0 for d in self.decay):
+            raise InvalidInput("retention needs positive sizes and one decay in (0, 1] for every head")
+        self.names = dict(q=q, k=k, v=v, g=g, o=o)
+        self.position = None
+        if position is not None:
+            if positions is None or position not in positions:
+                raise InvalidInput(f"retention names position encoding {position!r}, which the model does not define")
+            self.position = positions[position]
+            if getattr(self.position, "pairing", None) != "halves" or self.position.rot_dim > self.key_dim:
+                raise InvalidInput("retention turns channel i with channel i + rot_dim / 2 of a head: the position encoding must say so and fit")
+        self.qkvg = self.out = self.head_decay = None
+
+    def tensors(self):
+        H, d, e, n = self.heads, self.key_dim, self.value_dim, self.names
+        return [TensorSpec(n["q"], (H * d, self.width)), TensorSpec(n["k"], (H * d, self.width)), TensorSpec(n["v"], (H * e, self.width)),
+                TensorSpec(n["g"], (H * e, self.width)), TensorSpec(n["o"], (self.width, H * e))]
+
+    def check(self, rt):
+        if self.key_dim > 256:
+            raise Unsupported(f"the retention kernel takes up to 256 key channels a head, got {self.key_dim}")
+
+    def bind(self, weights, rt):
+        n = self.names
+        self.qkvg = Projection(torch.cat([weights[n[key]] for key in ("q", "k", "v", "g")], dim=0), rt)
+        self.out = Projection(weights[n["o"]], rt)
+        decay = torch.tensor(self.decay, dtype=torch.float64)
+        self.head_decay = torch.stack([decay, torch.log(decay)]).to(torch.float32).to(rt.device).contiguous()
+
+    def weight_bytes(self):
+        return self.qkvg.weight_bytes() + self.out.weight_bytes()
+
+    def cache_request(self):
+        return StateRequest((self.heads, self.key_dim, self.value_dim))
+
+    def forward(self, x, ctx, view, rt):
+        if view.read_only:
+            raise Unsupported("retention cannot read another layer's state")
+        H, d, e = self.heads, self.key_dim, self.value_dim
+        tokens = x.shape[0]
+        rows = self.qkvg(x, rt)
+        q, k = rows[:, :H * d], rows[:, H * d:2 * H * d]
+        v, g = rows[:, 2 * H * d:2 * H * d + H * e], rows[:, 2 * H * d + H * e:]
+        tables = self.position.rotary() if self.position is not None else None
+        rotation = (tables.cos, tables.sin, tables.rot_dim) if tables is not None else None
+        # (the keys' factor 1 / sqrt(d) rides on the queries: o is linear in both)
+        o = rt.ops.gla_scan(q, k, v, None, d ** -0.5, view.state, ctx, H, rt.empty(tokens, H * e, dtype=torch.float32),
+                            head_decay=self.head_decay, rotation=rotation)
+        gated = rt.ops.head_norm_gate(o, g, None, self.eps, H, rt.empty(tokens, H * e))
+        return self.out(gated, rt)
+
+
+class GatedDeltaRule(Mixer):
+    """The gated delta rule.  With H value heads of e channels on G query/key heads of d channels (value head h uses
+    query/key head h // (H / G)):
+
+        q, k, v = silu(conv(W_q h)), silu(conv(W_k h)), silu(conv(W_v h))     causal, per channel, ``taps`` wide, no bias
+        q <- q / sqrt(sum q^2 + 1e-6) / sqrt(d),   k <- k / sqrt(sum k^2 + 1e-6)          per head
+        beta = sigmoid(W_b h),   g = exp(-exp(A_log) softplus(W_a h + dt_bias))           one each a value head
+        S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q                   per head, S [d, e]
+        out = W_o (concat_h(o / rms(o) * w_norm) * silu(W_g h))
+
+    State per sequence: S [H, d, e] and the convolution's last ``taps`` - 1 inputs.  Queries, keys, values and the gate
+    leave one projection and one convolution; beta's and the decay's logits leave a second projection in 32-bit; unit
+    vectors, beta, decays, the recurrence and the norm are 32-bit under either runtime."""
+
+    graph_safe = True
+
+    def __init__(self, width, heads, qk_heads, key_dim, value_dim, taps, eps, q, k, v, q_conv, k_conv, v_conv, b, a, a_log, dt_bias,
+                 norm, g, o):
+        self.width, self.heads, self.qk_heads = int(width), int(heads), int(qk_heads)
+        self.key_dim, self.value_dim, self.taps, self.eps = int(key_dim), int(value_dim), int(taps), float(eps)
+        if min(self.heads, self.qk_heads, self.key_dim, self.value_dim, self.taps) <= 0 or self.heads % self.qk_heads:
+            raise InvalidInput("the gated delta rule needs positive sizes and value heads that divide among the query/key heads")
+        self.names = dict(q=q, k=k, v=v, q_conv=q_conv, k_conv=k_conv, v_conv=v_conv, b=b, a=a, a_log=a_log, dt_bias=dt_bias,
+                          norm=norm, g=g, o=o)
+        self.channels = 2 * self.qk_heads * self.key_dim + self.heads * self.value_dim  # what the convolution runs over
+
+    def tensors(self):
+        H, G, d, e, n = self.heads, self.qk_heads, self.key_dim, self.value_dim, self.names
+        return [
+            TensorSpec(n["q"], (G * d, self.width)), TensorSpec(n["q_conv"], (G * d, self.taps), init="conv_taps"),
+            TensorSpec(n["k"], (G * d, self.width)), TensorSpec(n["k_conv"], (G * d, self.taps), init="conv_taps"),
+            TensorSpec(n["v"], (H * e, self.width)), TensorSpec(n["v_conv"], (H * e, self.taps), init="conv_taps"),
+            TensorSpec(n["b"], (H, self.width)), TensorSpec(n["a_log"], (H,), init="small"), TensorSpec(n["norm"], (e,), init="gain"),
+            TensorSpec(n["a"], (H, self.width)), TensorSpec(n["dt_bias"], (H,), init="small"),
+            TensorSpec(n["g"], (H * e, self.width)), TensorSpec(n["o"], (self.width, H * e)),
+        ]
+
+    def check(self, rt):
+        if self.key_dim > 256 or self.taps > 16:
+            raise Unsupported(f"the gated delta rule's kernels take up to 256 key channels a head and 16 taps, got {self.key_dim} and {self.taps}")
+
+    def bind(self, weights, rt):
+        n = self.names
+        self.qkvg = Projection(torch.cat([weights[n[key]] for key in ("q", "k", "v", "g")], dim=0), rt)
+        self.conv = torch.cat([weights[n[key]] for key in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
+        self.ba = Projection(torch.cat([weights[n["b"]], weights[n["a"]]], dim=0), rt)
+        self.rate = torch.exp(weights[n["a_log"]].float()).contiguous()  # 32-bit, made once
+        self.dt_bias = weights[n["dt_bias"]].float().contiguous()
+        self.norm = weights[n["norm"]].contiguous()
+        self.out = Projection(weights[n["o"]], rt)
+
+    def weight_bytes(self):
+        small = sum(t.numel() * t.element_size() for t in (self.conv, self.rate, self.dt_bias, self.norm))
+        return small + sum(p.weight_bytes() for p in (self.qkvg, self.ba, self.out))
+
+    def cache_request(self):
+        return (StateRequest((self.heads, self.key_dim, self.value_dim)), StateRequest((self.taps - 1, self.channels)))
+
+    def forward(self, x, ctx, view, rt):
+        state, conv_state = view
+        if state.read_only:
+            raise Unsupported("the gated delta rule cannot read another layer's state")
+        H, e, tokens = self.heads, self.value_dim, x.shape[0]
+        rows = self.qkvg(x, rt)
+        ba = self.ba(x, rt, out_dtype=torch.float32)
+        qkv = rt.ops.conv_silu(rows, self.channels, self.conv, None, conv_state.state if self.taps > 1 else None, ctx,
+                               rt.empty(tokens, self.channels))
+        o = rt.ops.gated_delta(qkv, ba, self.rate, self.dt_bias, self.key_dim ** -0.5, state.state, ctx, H, self.qk_heads, self.key_dim,
+                               e, rt.empty(tokens, H * e, dtype=torch.float32))
+        gated = rt.ops.head_norm_gate(o, rows[:, self.channels:], self.norm, self.eps, H, rt.empty(tokens, H * e))
+        return self.out(gated, rt)
+
+
 class MinGRU(Mixer):
     """A gated recurrence whose gates read the current token only.  With C channels:
 
@@ -214,8 +357,10 @@ class MinGRU(Mixer):
 class SideBySide(Mixer):
     """Several mixers that read the same input; each output is divided by its
     root mean square over the model width and multiplied by a weight of its
-    own, and the result is the mean of these.  The cache gives each branch
-    what it asks for; the view is the tuple of their views.
+    own, and the result is the mean of these -- or, with ``scales`` in the
+    weights' place, the outputs are added as they are, each times its factor.
+    The cache gives each branch what it asks for; the view is the tuple of
+    their views.
 
     The branches do not depend on one another: the first runs on the stream
     the step is on, the others on a second stream of the same priority that
@@ -226,14 +371,17 @@ class SideBySide(Mixer):
 
     BESIDE_MOST_ROWS = 256  # steps of up to this many rows run the branches on two streams
 
-    def __init__(self, width, eps, branches, weights, positions=None):
+    def __init__(self, width, eps, branches, weights=None, positions=None, scales=None):
         from .base import build_part
 
-        if not 1 <= len(branches) <= 4 or len(weights) != len(branches):
-            raise InvalidInput("one to four branches side by side, each with a weight")
+        if (weights is None) == (scales is None):
+            raise InvalidInput("branches side by side are normed and weighted (weights), or added with a factor each (scales)")
+        if not 1 <= len(branches) <= 4 or len(weights if scales is None else scales) != len(branches):
+            raise InvalidInput("one to four branches side by side, each with a weight or a factor")
         self.width, self.eps = int(width), float(eps)
         self.branches = [build_part("mixer", description, positions=positions) for description in branches]
-        self.weight_names = list(weights)
+        self.scales = None if scales is None else [float(value) for value in scales]
+        self.weight_names = list(weights or [])
         self.weights = None
         self.graph_safe = all(getattr(branch, "graph_safe", False) for branch in self.branches)
         self._beside = None  # the second stream, made at the first step
@@ -269,7 +417,7 @@ class SideBySide(Mixer):
         return [buffer for branch in self.branches for buffer in branch.held_buffers(rt)]
 
     def _run(self, branch, x, ctx, branch_view, rt):
-        if getattr(branch, "can_leave_bias", False):
+        if self.scales is None and getattr(branch, "can_leave_bias", False):
             return branch.forward(x, ctx, branch_view, rt, bias_later=True), branch.output_bias
         return branch.forward(x, ctx, branch_view, rt), None
 
@@ -293,6 +441,8 @@ class SideBySide(Mixer):
             for index in range(count):
                 results[index] = self._run(self.branches[index], x, ctx, view[index], rt)
         outputs, biases = [r[0] for r in results], [r[1] for r in results]
+        if self.scales is not None:
+            return rt.ops.branch_sum(outputs, self.scales, rt.empty(x.shape[0], self.width))
         return rt.ops.branch_mean(outputs, self.weights, biases, self.eps, rt.empty(x.shape[0], self.width))
 
 
@@ -313,5 +463,7 @@ register_init_rule("decay_bias", lambda spec, generator, dtype: (2.0 + _noise(sp
 
 register_part("mixer", "selective_scan", SelectiveScan)
 register_part("mixer", "gated_linear_attention", GatedLinearAttention)
+register_part("mixer", "retention", Retention)
+register_part("mixer", "gated_delta_rule", GatedDeltaRule)
 register_part("mixer", "min_gru", MinGRU)
 register_part("mixer", "side_by_side", SideBySide)

@@ -45,6 +45,12 @@ reading an earlier layer's keys; minGRU; PolyNorm and routed feed-forwards;
 norms on the sublayers' outputs only) beside a Mutedra of windowed-attention
 layers of the same width, layers, heads, window, inner size and vocabulary.
 
+``--workload mafalorn`` measures the Mafalorn design (retention; grouped
+attention whose values are its keys beside the gated delta rule; attention
+over a cached latent in a window with a gate element by element; experts chosen
+among groups; RMS norms before and after every sublayer) beside a Zifunex of
+the same width, layers, heads, state sizes, inner size and vocabulary.
+
 Peaks used for the fractions are the published MI355X ones: HBM 8 TB/s; dense
 matrix rate 2.5 PFLOP/s for bfloat16, 157.3 TFLOP/s for 32-bit.
 """
@@ -226,7 +232,8 @@ def prefill_run(shape, rng, tokens=2048):
     del engine
     torch.cuda.empty_cache()
     seconds = sorted(times[3:])[3]  # the median of seven runs of a shape that has come before (and is captured, where it is)
-    flops = {"Zifunex": zifunex_step_flops, "Mutedra": mutedra_step_flops, "Robopel": robopel_step_flops}.get(shape.config.get("architecture"), step_flops)(
+    flops = {"Zifunex": zifunex_step_flops, "Mutedra": mutedra_step_flops, "Robopel": robopel_step_flops,
+             "Mafalorn": mafalorn_step_flops}.get(shape.config.get("architecture"), step_flops)(
         shape.config, [tokens], 1)
     return {"value": round(tokens / seconds, 1), "tokens": tokens, "ms": round(1000.0 * seconds, 3),
             "frac": round(flops / seconds / FLOP_PEAK[shape.dtype], 5), "first_ms": round(1000.0 * times[0], 3)}
@@ -454,6 +461,90 @@ def robopel_twin_config(sizes):
             "logit_softcap": 30.0, "layers": [layer] * len(ROBOPEL_LAYERS), "loop": {"start": 0, "stop": len(ROBOPEL_LAYERS), "times": 1}}
 
 
+# Mafalorn at two sets of layer sizes: R = retention, P = attention whose values are its keys beside the gated delta
+# rule, L = attention over a latent in a window; every layer with experts chosen among two groups.  Per set: retention
+# (heads, key channels, value channels), the softmax side (query heads, key/value heads, channels, turned channels), the
+# delta rule (value heads, query/key heads, key channels, value channels, taps), the latent (heads, plain key
+# channels, turned channels, value channels, latent, window), experts (experts, chosen, identity outputs, inner size).
+MAFALORN_SETS = {
+    "w1024": dict(width=1024, retention=(4, 128, 256), softmax=(16, 4, 64, 64), delta=(8, 4, 64, 128, 4), latent=(16, 64, 32, 64, 128, 512),
+                  moe=(8, 2, 2, 352)),
+    "w2048": dict(width=2048, retention=(8, 128, 256), softmax=(16, 4, 128, 64), delta=(16, 8, 128, 128, 4), latent=(16, 128, 64, 128, 192, 1024),
+                  moe=(8, 2, 2, 704)),
+}
+MAFALORN_LAYERS = "RPRLRPRL"
+
+
+def mafalorn_config(sizes):
+    r_heads, r_dim, r_vdim = sizes["retention"]
+    heads, kv_heads, dim, turned = sizes["softmax"]
+    d_heads, d_qk, d_dim, d_vdim, taps = sizes["delta"]
+    l_heads, l_dim, l_rot, l_vdim, rank, window = sizes["latent"]
+    experts, top, identity, expert_ff = sizes["moe"]
+    mlp = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "identity": identity,
+                                                                  "groups": {"count": 2, "keep": 1}}}
+    kinds = {
+        "R": {"type": "retention", "mlp": mlp, "mixer": {
+            "heads": r_heads, "dim": r_dim, "vdim": r_vdim, "decay": [1.0 - 2.0 ** (-5 - h) for h in range(r_heads)],
+            "rot": {"dims": r_dim, "base": 10000.0}}},
+        "P": {"type": "parallel", "mlp": mlp, "mixer": {
+            "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                     "rot": {"dims": turned, "base": 10000.0, "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}},
+            "right": {"heads": d_heads, "kv_heads": d_qk, "dim": d_dim, "vdim": d_vdim, "conv": taps},
+            "left_scale": 0.7, "right_scale": 0.7}},
+        "L": {"type": "latent_attention", "mlp": mlp, "mixer": {
+            "heads": l_heads, "dim": l_dim, "rot_dim": l_rot, "vdim": l_vdim, "kv_rank": rank, "scale": (l_dim + l_rot) ** -0.5,
+            "rot": {"dims": l_rot, "base": 10000.0}, "mask": {"size": window}}},
+    }
+    return {"architecture": "Mafalorn", "vocab": ZIFUNEX_VOCAB, "width": sizes["width"], "norm": {"eps": 1e-6}, "logit_scale": 0.5,
+            "layers": [kinds[kind] for kind in MAFALORN_LAYERS]}
+
+
+def mafalorn_step_flops(config, tokens_per_sequence, wanted_rows):
+    """Multiply-adds x2 of one step over whole prompts from empty slots: the projections, the two recurrences, the
+    softmax side's keys, a window's latents, and of the experts those that a token has chosen (the library multiplies
+    all of them)."""
+    w = config["width"]
+    total = 0
+    for n in tokens_per_sequence:
+        for layer in config["layers"]:
+            m = layer["mixer"]
+            if layer["type"] == "retention":
+                hd, he = m["heads"] * m["dim"], m["heads"] * m["vdim"]
+                total += 2 * ((2 * hd + 3 * he) * w + 2 * m["heads"] * m["dim"] * m["vdim"]) * n
+            elif layer["type"] == "parallel":
+                a, r = m["left"], m["right"]
+                per_token = (2 * a["heads"] + a["kv_heads"]) * a["dim"] * w
+                per_token += (2 * r["kv_heads"] * r["dim"] + 3 * r["heads"] * r["vdim"] + 2 * r["heads"]) * w + 3 * r["heads"] * r["dim"] * r["vdim"]
+                total += 2 * per_token * n + 2 * a["heads"] * 2 * a["dim"] * n * (n + 1) // 2
+            else:
+                per_token = (m["heads"] * (m["dim"] + m["rot_dim"]) + m["kv_rank"] + m["rot_dim"] + 2 * m["heads"] * m["vdim"]) * w
+                per_token += m["heads"] * m["kv_rank"] * (m["dim"] + m["vdim"])
+                size = (m.get("mask") or {}).get("size") or n
+                keys = sum(min(i + 1, size) for i in range(n))
+                total += 2 * per_token * n + 2 * m["heads"] * (2 * m["kv_rank"] + m["rot_dim"]) * keys
+            mlp = layer["mlp"]
+            if mlp is not None:
+                router = mlp["router"]
+                total += 2 * (3 * w * mlp["expert"]["ff"] * router["top"] + (router["experts"] + router.get("identity", 0)) * w) * n
+    return total + 2 * wanted_rows * w * config["vocab"]
+
+
+def mafalorn_twin_config(sizes):
+    """The closest model the library had: a Zifunex whose gated linear attention has retention's heads, whose attention
+    has the softmax side's, whose scan stands where the delta rule and the latent do, and whose feed-forward's inner
+    size is all the experts' together: the same width, layers and vocabulary."""
+    r_heads, r_dim, r_vdim = sizes["retention"]
+    heads, kv_heads, dim, _ = sizes["softmax"]
+    experts, _, _, expert_ff = sizes["moe"]
+    twin = dict(width=sizes["width"], ff=experts * expert_ff, attention=(heads, kv_heads, dim, dim), scan=(2 * sizes["width"], 16, sizes["width"] // 16, 4),
+                gla=(r_heads, r_dim, r_vdim, 32), streams=1)
+    config = zifunex_config(twin)
+    side_by_side, linear = config["layers"][0], config["layers"][2]
+    config["layers"] = [linear if kind == "R" else side_by_side for kind in MAFALORN_LAYERS]
+    return config
+
+
 def design_run(args, rng, design, sets, config_of, twin_of, twin="llama"):
     """Each set of sizes: the design's model and its Llama twin, a prompt of 2,048 tokens and decode at batch 1, 8, 64."""
     import torch
@@ -506,7 +597,7 @@ def main() -> int:
     parser.add_argument("--no-other-shapes", action="store_true", help="points of the headline's shape only")
     parser.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the decode batches")
     parser.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the decode batches (within the context)")
-    parser.add_argument("--workload", choices=["tinyllama-ragged", "zifunex", "mutedra", "robopel"], help="run this workload alone")
+    parser.add_argument("--workload", choices=["tinyllama-ragged", "zifunex", "mutedra", "robopel", "mafalorn"], help="run this workload alone")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -548,6 +639,18 @@ def main() -> int:
             "ms_per_step": head["ms_per_step"], "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic: random weights from a seed, uniform-random token ids",
             "config": {"model": "Robopel, 8 layers of width 2048 (decode at batch 8)", "sets": ROBOPEL_SETS, "layers": ROBOPEL_LAYERS,
+                       "vocab": ZIFUNEX_VOCAB, "context": ZIFUNEX_CONTEXT, "prompt_min": args.prompt_min, "prompt_max": args.prompt_max},
+            "models": models, "env": environment()}))
+        return 0
+    if args.workload == "mafalorn":
+        models = design_run(args, rng, "mafalorn", MAFALORN_SETS, mafalorn_config, mafalorn_twin_config, twin="zifunex")
+        head = models["mafalorn-w2048"]["decode_b8"]
+        print(json.dumps({
+            "metric": "Mafalorn at two sets of layer sizes beside a Zifunex of the same sizes: prefill of 2,048 tokens, decode at batch 1, 8, 64",
+            "value": head["tokens_per_second"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": head["ms_per_step"], "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic: random weights from a seed, uniform-random token ids",
+            "config": {"model": "Mafalorn, 8 layers of width 2048 (decode at batch 8)", "sets": MAFALORN_SETS, "layers": MAFALORN_LAYERS,
                        "vocab": ZIFUNEX_VOCAB, "context": ZIFUNEX_CONTEXT, "prompt_min": args.prompt_min, "prompt_max": args.prompt_max},
             "models": models, "env": environment()}))
         return 0

@@ -60,7 +60,9 @@ PREBUILT_WIDE_VALUES = ("attn_hd7v5c", "attn_hd32v16c", "attn_hd16v48c", "attn_h
                         # sizes of the measurements
                         "attn_hd32v16cx", "attn_hd32v16xp", "attn_hd32v16cxp", "attn_hd16v48cx", "attn_hd16v48xp", "attn_hd16v48cxp",
                         "attn_hd24v40x", "attn_hd24v40cx", "attn_hd24v40xp", "attn_hd24v40cxp", "attn_hd16cx", "attn_hd16xp", "attn_hd16cxp",
-                        "attn_hd20v12xp", "attn_hd32xp", "attn_hd64cxp", "attn_hd128cxp")
+                        "attn_hd20v12xp", "attn_hd32xp", "attn_hd64cxp", "attn_hd128cxp",
+                        # latents as the one key/value head without any extras, in a window or not: the tests' sizes and the measurements'
+                        "attn_hd48v40", "attn_hd64v48", "attn_hd32v24", "attn_hd20v16", "attn_hd160v128", "attn_hd256v192")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

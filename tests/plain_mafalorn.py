@@ -91,8 +91,10 @@ def retention(h, w, sizes, eps, rnd=identity, first=0, state=None):
     n = h.shape[0]
     heads, dim, vdim = sizes["heads"], sizes["dim"], sizes["vdim"]
     positions = torch.arange(first, first + n)
-    q = turn(rnd(h @ w["q"].T).view(n, heads, dim), positions, sizes["rot"], "halves")
-    k = turn(rnd(h @ w["k"].T).view(n, heads, dim), positions, sizes["rot"], "halves") * dim ** -0.5
+    q, k = rnd(h @ w["q"].T).view(n, heads, dim), rnd(h @ w["k"].T).view(n, heads, dim)
+    if sizes.get("rot") is not None:
+        q, k = turn(q, positions, sizes["rot"], "halves"), turn(k, positions, sizes["rot"], "halves")
+    k = k * dim ** -0.5
     v = rnd(h @ w["v"].T).view(n, heads, vdim)
     gate = silu(rnd(h @ w["g"].T))
     decay = torch.tensor(sizes["decay"], dtype=h.dtype)[:, None, None]
@@ -185,7 +187,7 @@ def latent_attention(h, w, sizes, eps, rnd=identity):
     down = h @ w["dkv"].T
     c = rnd(rms_norm(down[:, :rank], w["dkv.norm"], eps))
     shared = down[:, rank:].view(n, 1, rot_dim)
-    q_plain, q_rot, k_rot = q[..., :dim], q[..., dim:], shared
+    q_plain, q_rot, k_rot = q[..., :dim], q[..., dim:], rnd(shared)
     if rot_dim:
         rot = dict(sizes["rot"], dims=rot_dim)
         q_rot, k_rot = turn(q_rot, positions, rot, "neighbours"), rnd(turn(shared, positions, rot, "neighbours"))
@@ -265,10 +267,28 @@ def forward(config, weights, tokens, rnd=identity, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     h = rnd(rms_norm(x, w["final.norm"], eps))
-    return (h @ w["head"].T) * config["logit_scale"]
+    return (h @ w["head"].T) * config.get("logit_scale", 1.0)
 
 
 def load(folder):
     with open(os.path.join(folder, "config.json")) as handle:
         config = json.load(handle)
     return config, load_file(os.path.join(folder, "model.safetensors"))
+
+
+class PlainMafalorn:
+    """The whole model over one sequence from its first token, from a folder with config.json and model.safetensors."""
+
+    def __init__(self, folder):
+        self.config, self.weights = load(folder)
+
+    def logits(self, ids, rnd=identity, stream_after=None):
+        """Logits [tokens, vocab]; ``stream_after`` (a list) gets the stream after every layer."""
+        return forward(self.config, self.weights, list(ids), rnd, stream_after)
+
+    def greedy(self, ids, count):
+        ids, out = list(ids), []
+        for _ in range(count):
+            out.append(int(self.logits(ids)[-1].argmax()))
+            ids.append(out[-1])
+        return out

@@ -166,6 +166,56 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const void* __restric
   }
 }
 
+// The same on the matrix cores for bfloat16 rows and maps with K a multiple of 8, up to kHeadsLinearMostK: a block takes 16
+// rows of one head; each of its 4 waves keeps the rows' K in operand registers and takes every fourth strip of 16
+// outputs, whose weights come straight from memory (a head's map is small and read by every block of the head: it
+// stays in the caches).  v_mfma_f32_16x16x32_bf16 with the map's rows as the first operand: lane l holds outputs
+// 4 * (l / 16) .. + 3 of row l % 16, four consecutive outputs of one row, gated and stored together.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_m;
+typedef __attribute__((ext_vector_type(4))) float f32x4_m;
+constexpr int kHeadsLinearMostK = 512;
+
+template <int CHUNKS>
+__global__ __launch_bounds__(256) void heads_linear_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                const float* __restrict__ gate, bf16_t* __restrict__ out, int tokens,
+                                                                int heads, int n, int k) {
+  const int head = blockIdx.y, row0 = blockIdx.x * 16;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int r = lane % 16, group = lane / 16;
+  const int token = min(row0 + r, tokens - 1);
+  bf16x8_m rows[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int at = c * 32 + group * 8;
+    bf16x8_m v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (__bf16)0.0f;
+    if (at < k) v = *(const bf16x8_m*)(x + ((size_t)token * heads + head) * k + at);
+    rows[c] = v;
+  }
+  for (int strip = wave; strip * 16 < n; strip += 4) {
+    const int o = min(strip * 16 + r, n - 1);
+    const bf16_t* map = w + ((size_t)head * n + o) * k;
+    f32x4_m acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const int at = c * 32 + group * 8;
+      bf16x8_m v;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = (__bf16)0.0f;
+      if (at < k) v = *(const bf16x8_m*)(map + at);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, rows[c], acc, 0, 0, 0);
+    }
+    if (row0 + r >= tokens) continue;
+    const int first = strip * 16 + group * 4;  // this lane's four outputs of row r
+    const size_t at = ((size_t)(row0 + r) * heads + head) * n + first;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (first + e < n) out[at + e] = (__bf16)(gate ? acc[e] * gate[at + e] : acc[e]);
+    }
+  }
+}
+
 unsigned blocks_for(size_t total) {
   size_t blocks = (total + 255) / 256;
   return (unsigned)(blocks > 65536 ? 65536 : blocks);
@@ -245,11 +295,26 @@ extern "C" int nnis_heads_linear(const void* x, int x_dtype, const void* w, int 
   NNIS_REQUIRE(x && w && out && tokens >= 0 && heads > 0 && heads <= 65535 && n > 0 && k > 0, "heads_linear: bad arguments");
   NNIS_REQUIRE((size_t)k * sizeof(float) <= 48 * 1024, "heads_linear: rows of up to 12288 channels a head, got %d", k);
   if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (x_dtype == NNIS_BF16 && w_dtype == NNIS_BF16 && out_dtype == NNIS_BF16 && k % 8 == 0 && k <= kHeadsLinearMostK &&
+      (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0) {
+    const dim3 tiles((tokens + 15) / 16, heads);
+    const int chunks = (k + 31) / 32;
+#define NNIS_HEADS_LINEAR(C_)   hipLaunchKernelGGL((heads_linear_mfma_kernel<C_>), tiles, dim3(256), 0, s, (const bf16_t*)x, (const bf16_t*)w, gate, (bf16_t*)out, tokens, heads, n, k)
+    if (chunks <= 2) NNIS_HEADS_LINEAR(2);
+    else if (chunks <= 4) NNIS_HEADS_LINEAR(4);
+    else if (chunks <= 6) NNIS_HEADS_LINEAR(6);
+    else if (chunks <= 8) NNIS_HEADS_LINEAR(8);
+    else if (chunks <= 12) NNIS_HEADS_LINEAR(12);
+    else NNIS_HEADS_LINEAR(16);
+#undef NNIS_HEADS_LINEAR
+    NNIS_LAUNCH_CHECK("heads_linear");
+    return 0;
+  }
   // several rows a block where they fit 48 KB of LDS and the step has rows enough
   const int rows = tokens >= 64 && (size_t)8 * k * 4 <= 49152 ? 8 : (tokens >= 4 && (size_t)4 * k * 4 <= 49152 ? 4 : 1);
   const dim3 grid((tokens + rows - 1) / rows, heads);
   const size_t lds = (size_t)rows * k * sizeof(float);
-  hipStream_t s = (hipStream_t)stream;
   if (rows == 8) hipLaunchKernelGGL((heads_linear_kernel<8>), grid, dim3(256), lds, s, x, x_dtype, w, w_dtype, gate, out, out_dtype, tokens, heads, n, k);
   else if (rows == 4) hipLaunchKernelGGL((heads_linear_kernel<4>), grid, dim3(256), lds, s, x, x_dtype, w, w_dtype, gate, out, out_dtype, tokens, heads, n, k);
   else hipLaunchKernelGGL((heads_linear_kernel<1>), grid, dim3(256), lds, s, x, x_dtype, w, w_dtype, gate, out, out_dtype, tokens, heads, n, k);

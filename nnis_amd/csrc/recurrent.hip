@@ -894,10 +894,15 @@ extern "C" int nnis_min_gru(const void* rows, int dtype, int stride, const void*
 //   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
 // with q and k unit vectors over a head's channels (x / sqrt(sum x^2 + unit_eps); q also times q_scale), beta =
 // sigmoid(b), g = exp(-rate_h * softplus(a + dt_bias_h)).  Query/key head of value head h: h / (heads / groups).
-// The columns of S do not meet: a block takes one head of one sequence and a slab of value columns; a thread keeps
-// 16 key rows of one column, the threads of a column sit 64 / GROUPS lanes apart in one wave and add their parts of
-// S^T k and S^T q by lane exchanges.  Tokens come through LDS a chunk at a time: a wave a token makes the unit
-// vectors, a thread a token the gates.  Everything but the rows' storage type is 32-bit; o is left raw, in 32-bit.
+//
+// Two kernels.  delta_prepare_kernel, a wave a (token, query/key head): the unit vectors in 32-bit, their product q . k,
+// and, a thread a (token, value head), g and beta.  gated_delta_kernel, the recurrence: the columns of S do not meet, so
+// a block takes one head of one sequence and a slab of value columns; a thread keeps 8 key rows of one column, and the
+// threads of a column are neighbouring lanes, so that their parts of a sum meet by lane moves inside a row of 16
+// lanes.  Written on the state before the token, a token needs ONE round of sums, of two numbers side by side:
+//   a = S^T k,  b = S^T q  (before the token);   u = beta (v - g a);   o = g b + (q . k) u;   S <- g S + k u^T
+// Tokens come through LDS a chunk at a time, copied by the whole block.  Everything but the rows' storage type is
+// 32-bit; o is left raw, in 32-bit.
 // -----------------------------------------------------------------------------
 namespace {
 
@@ -908,21 +913,102 @@ struct DeltaArgs {
   const float* rate;     // [heads]: exp(A_log)
   const float* dt_bias;  // [heads]
   float q_scale, unit_eps;
-  float* state;  // [slots, heads, key_dim, value_dim]
+  float* unit;   // [tokens, groups, 2, key_dim]: q then k, unit vectors
+  float* gates;  // [tokens, heads, 2]: g, beta;  behind them [tokens, groups]: q . k
+  float* state;  // [slots, heads, value_dim, key_dim]: column by column
   const int* seq_slot;
   const int* seq_start;
-  int heads, groups, key_dim, value_dim;
+  int tokens, heads, groups, key_dim, value_dim;
   int chunk;
   float* out;  // [tokens, heads * value_dim]
 };
 
+__global__ __launch_bounds__(256) void delta_prepare_kernel(DeltaArgs a) {
+  const int d = a.key_dim;
+  const int item = blockIdx.x * 4 + threadIdx.x / kWave;  // (token, query/key head)
+  const int lane = threadIdx.x % kWave;
+  const int items = a.tokens * a.groups;
+  if (item < items) {
+    const int t = item / a.groups, qk_head = item % a.groups;
+    const size_t q_at = (size_t)t * a.stride + (size_t)qk_head * d;
+    const size_t k_at = q_at + (size_t)a.groups * d;
+    float sq = 0.0f, sk = 0.0f;
+    for (int ch = lane; ch < d; ch += kWave) {
+      const float q = load_as_f32(a.rows, a.dtype, q_at + ch), k = load_as_f32(a.rows, a.dtype, k_at + ch);
+      sq = fmaf(q, q, sq);
+      sk = fmaf(k, k, sk);
+    }
+    const float inv_q = (1.0f / sqrtf(wave_sum(sq) + a.unit_eps)) * a.q_scale;
+    const float inv_k = 1.0f / sqrtf(wave_sum(sk) + a.unit_eps);
+    float* into = a.unit + (size_t)item * 2 * d;
+    float qk = 0.0f;
+    for (int ch = lane; ch < d; ch += kWave) {
+      const float q = load_as_f32(a.rows, a.dtype, q_at + ch) * inv_q, k = load_as_f32(a.rows, a.dtype, k_at + ch) * inv_k;
+      into[ch] = q;
+      into[d + ch] = k;
+      qk = fmaf(q, k, qk);
+    }
+    qk = wave_sum(qk);
+    if (lane == 0) a.gates[(size_t)a.tokens * a.heads * 2 + item] = qk;
+  }
+  // g and beta: a thread a (token, value head), dealt over the whole launch
+  const int per_block = blockDim.x;
+  for (int i = blockIdx.x * per_block + threadIdx.x; i < a.tokens * a.heads; i += gridDim.x * per_block) {
+    const int t = i / a.heads, head = i % a.heads;
+    const float* ba = a.ba + (size_t)t * 2 * a.heads;
+    const float z = ba[a.heads + head] + a.dt_bias[head];
+    const float soft = z > 20.0f ? z : log1pf(expf(z));
+    a.gates[2 * (size_t)i] = expf(-a.rate[head] * soft);
+    a.gates[2 * (size_t)i + 1] = 1.0f / (1.0f + expf(-ba[head]));
+  }
+}
+
+// the sum of x over the GROUPS neighbouring lanes of a column (GROUPS a power of two up to 32): moves inside a row of
+// 16 lanes, and one exchange between two rows for 32
+template <int GROUPS>
+__device__ __forceinline__ float column_sum(float x) {
+  if (GROUPS >= 2) x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));   // lanes 1 0 3 2
+  if (GROUPS >= 4) x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));   // lanes 2 3 0 1
+  if (GROUPS >= 8) x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));  // a half row mirrored
+  if (GROUPS >= 16) x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x140, 0xF, 0xF, true)); // a row mirrored
+  if (GROUPS >= 32) x += __shfl_xor(x, 16, kWave);
+  return x;
+}
+
+// what a thread needs of a token: its 8 key rows of q and k, the token's g, beta and q . k, its column's v
+struct DeltaToken {
+  float4 k[2], q[2], gate;
+  float v;
+};
+
+template <int GROUPS>
+__device__ __forceinline__ DeltaToken delta_token(const float* qk, const float* vs, const float* gs, int j, int group, int col_in_block,
+                                                  int cols) {
+  constexpr int kPad = GROUPS * 8;
+  DeltaToken t;
+  const float* qj = qk + j * 2 * kPad + group * 8;
+  const float* kj = qj + kPad;
+  t.k[0] = *(const float4*)kj;
+  t.k[1] = *(const float4*)(kj + 4);
+  t.q[0] = *(const float4*)qj;
+  t.q[1] = *(const float4*)(qj + 4);
+  t.gate = *(const float4*)(gs + 4 * j);
+  t.v = vs[j * cols + col_in_block];
+  return t;
+}
+
+// A thread keeps 8 key rows of one column; the GROUPS threads of a column are neighbouring lanes.  The state lies
+// column by column, [slots, heads, value_dim, key_dim]: a column's threads read and write consecutive memory.
+// A chunk's numbers are all asked for from memory before any of them is waited for.
 template <int GROUPS>
 __global__ __launch_bounds__(256) void gated_delta_kernel(DeltaArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int kPad = GROUPS * 16;            // key rows as the threads see them (rows beyond key_dim are zero)
+  constexpr int kPad = GROUPS * 8;             // key rows as the threads see them (rows beyond key_dim are zero)
   constexpr int kPer = kWave / GROUPS;         // columns of a wave
   constexpr int kCols = 4 * kPer;              // columns of a block
-  constexpr int kEach = (kPad + kWave - 1) / kWave;  // channels a lane takes of a vector
+  constexpr int kChunk = GROUPS >= 32 ? 16 : 32;  // tokens staged at a time
+  constexpr int kQkLoads = (kChunk * 2 * kPad / 4 + 255) / 256;  // 16-byte loads a thread makes of a chunk's q and k
+  constexpr int kVLoads = (kChunk * kCols + 255) / 256;
   const int b = blockIdx.z, head = blockIdx.y;
   const int slot = a.seq_slot[b];
   if (slot < 0) return;
@@ -931,134 +1017,141 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(DeltaArgs a) {
   const int d = a.key_dim, e = a.value_dim;
   const int qk_head = head / (a.heads / a.groups);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int group = lane / kPer;
-  const int col_in_block = wave * kPer + lane % kPer;
+  const int group = lane % GROUPS;             // which 8 key rows
+  const int col_in_block = wave * kPer + lane / GROUPS;
   const int col = blockIdx.x * kCols + col_in_block;
   const bool live = col < e;
-  float* qs = lds;                     // [chunk][kPad]
-  float* ks = qs + a.chunk * kPad;     // [chunk][kPad]
-  float* vs = ks + a.chunk * kPad;     // [chunk][kCols]
-  float* gs = vs + a.chunk * kCols;    // [chunk][2]: g, beta
-  float* state = a.state + (((size_t)slot * a.heads + head) * d) * e + (live ? col : 0);
-  float S[16];
+  float* qk = lds;                        // [chunk][2][kPad]: a token's q, then its k
+  float* vs = qk + kChunk * 2 * kPad;     // [chunk][kCols]
+  float* gs = vs + kChunk * kCols;        // [chunk][4]: g, beta, q . k
+  float* state = a.state + (((size_t)slot * a.heads + head) * e + (live ? col : 0)) * d + group * 8;
+  float S[8];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = group * 16 + r;
-    S[r] = live && row < d ? state[(size_t)row * e] : 0.0f;
-  }
-  const size_t k_col0 = (size_t)a.groups * d;
+  for (int r = 0; r < 8; ++r) S[r] = live && group * 8 + r < d ? state[r] : 0.0f;
   const size_t v_col0 = 2 * (size_t)a.groups * d;
-  for (int t0 = begin; t0 < end; t0 += a.chunk) {
-    const int count = min(a.chunk, end - t0);
-    __syncthreads();  // the chunk before has been read
-    // unit vectors: a wave a (token, query or key)
-    for (int item = wave; item < 2 * count; item += 4) {
-      const int j = item >> 1, is_key = item & 1;
-      const size_t at = (size_t)(t0 + j) * a.stride + (is_key ? k_col0 : 0) + (size_t)qk_head * d;
-      float x[kEach];
-      float ss = 0.0f;
+  const float* qk_dots = a.gates + (size_t)a.tokens * a.heads * 2;
+  const bool whole = d == kPad;  // a token's q and k are what LDS holds of it: copied 16 bytes at a time
+  for (int t0 = begin; t0 < end; t0 += kChunk) {
+    const int count = min(kChunk, end - t0);
+    float4 qk_in[kQkLoads];
+    float v_in[kVLoads];
+    float gate_in[3] = {0.0f, 0.0f, 0.0f};
+    if (whole) {
 #pragma unroll
-      for (int i = 0; i < kEach; ++i) {
-        const int ch = i * kWave + lane;
-        x[i] = ch < d ? load_as_f32(a.rows, a.dtype, at + ch) : 0.0f;
-        ss = fmaf(x[i], x[i], ss);
-      }
-      const float inv = (1.0f / sqrtf(wave_sum(ss) + a.unit_eps)) * (is_key ? 1.0f : a.q_scale);
-      float* into = (is_key ? ks : qs) + j * kPad;
-#pragma unroll
-      for (int i = 0; i < kEach; ++i) {
-        const int ch = i * kWave + lane;
-        if (ch < kPad) into[ch] = x[i] * inv;
+      for (int it = 0; it < kQkLoads; ++it) {
+        const int f = threadIdx.x + it * 256, j = f / (kPad / 2), w = f % (kPad / 2);
+        if (f < count * (kPad / 2)) qk_in[it] = *(const float4*)(a.unit + ((size_t)(t0 + j) * a.groups + qk_head) * 2 * d + 4 * w);
       }
     }
-    for (int i = threadIdx.x; i < count * kCols; i += blockDim.x) {
+#pragma unroll
+    for (int it = 0; it < kVLoads; ++it) {
+      const int i = threadIdx.x + it * 256;
       const int t = t0 + i / kCols, cl = blockIdx.x * kCols + i % kCols;
-      vs[i] = cl < e ? load_as_f32(a.rows, a.dtype, (size_t)t * a.stride + v_col0 + (size_t)head * e + cl) : 0.0f;
+      v_in[it] = i < count * kCols && cl < e ? load_as_f32(a.rows, a.dtype, (size_t)t * a.stride + v_col0 + (size_t)head * e + cl) : 0.0f;
     }
     if ((int)threadIdx.x < count) {
-      const float* ba = a.ba + (size_t)(t0 + threadIdx.x) * 2 * a.heads;
-      const float z = ba[a.heads + head] + a.dt_bias[head];
-      const float soft = z > 20.0f ? z : log1pf(expf(z));
-      gs[2 * threadIdx.x] = expf(-a.rate[head] * soft);
-      gs[2 * threadIdx.x + 1] = 1.0f / (1.0f + expf(-ba[head]));
+      const int t = t0 + threadIdx.x;
+      gate_in[0] = a.gates[2 * ((size_t)t * a.heads + head)];
+      gate_in[1] = a.gates[2 * ((size_t)t * a.heads + head) + 1];
+      gate_in[2] = qk_dots[(size_t)t * a.groups + qk_head];
+    }
+    __syncthreads();  // the chunk before has been read
+    if (whole) {
+#pragma unroll
+      for (int it = 0; it < kQkLoads; ++it) {
+        const int f = threadIdx.x + it * 256;
+        if (f < count * (kPad / 2)) *(float4*)(qk + 4 * f) = qk_in[it];
+      }
+    } else {
+      for (int i = threadIdx.x; i < count * 2 * kPad; i += blockDim.x) {
+        const int j = i / (2 * kPad), ch = i % kPad, is_key = (i / kPad) & 1;
+        qk[i] = ch < d ? a.unit[((size_t)(t0 + j) * a.groups + qk_head) * 2 * d + is_key * d + ch] : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < kVLoads; ++it) {
+      const int i = threadIdx.x + it * 256;
+      if (i < count * kCols) vs[i] = v_in[it];
+    }
+    if ((int)threadIdx.x < count) {
+      gs[4 * threadIdx.x] = gate_in[0];
+      gs[4 * threadIdx.x + 1] = gate_in[1];
+      gs[4 * threadIdx.x + 2] = gate_in[2];
     }
     __syncthreads();
+    // a token's numbers are read from LDS while the token before is worked on
+    DeltaToken next = delta_token<GROUPS>(qk, vs, gs, 0, group, col_in_block, kCols);
     for (int j = 0; j < count; ++j) {
-      const float g = gs[2 * j], beta = gs[2 * j + 1];
-      const float v = vs[j * kCols + col_in_block];
-      const float* qj = qs + j * kPad + group * 16;
-      const float* kj = ks + j * kPad + group * 16;
-      float kv[16];
-      float dot = 0.0f;
+      const DeltaToken now = next;
+      if (j + 1 < count) next = delta_token<GROUPS>(qk, vs, gs, j + 1, group, col_in_block, kCols);
+      const float kv[8] = {now.k[0].x, now.k[0].y, now.k[0].z, now.k[0].w, now.k[1].x, now.k[1].y, now.k[1].z, now.k[1].w};
+      const float qv[8] = {now.q[0].x, now.q[0].y, now.q[0].z, now.q[0].w, now.q[1].x, now.q[1].y, now.q[1].z, now.q[1].w};
+      float dot_k[2] = {0.0f, 0.0f}, dot_q[2] = {0.0f, 0.0f};
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const float4 k4 = *(const float4*)(kj + 4 * r4);
-        kv[4 * r4] = k4.x; kv[4 * r4 + 1] = k4.y; kv[4 * r4 + 2] = k4.z; kv[4 * r4 + 3] = k4.w;
+      for (int r = 0; r < 8; r += 2) {
+        dot_k[0] = fmaf(S[r], kv[r], dot_k[0]);
+        dot_k[1] = fmaf(S[r + 1], kv[r + 1], dot_k[1]);
+        dot_q[0] = fmaf(S[r], qv[r], dot_q[0]);
+        dot_q[1] = fmaf(S[r + 1], qv[r + 1], dot_q[1]);
       }
+      const float with_k = column_sum<GROUPS>(dot_k[0] + dot_k[1]);
+      const float with_q = column_sum<GROUPS>(dot_q[0] + dot_q[1]);
+      const float g = now.gate.x;
+      const float u = now.gate.y * (now.v - g * with_k);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        S[r] *= g;
-        dot = fmaf(S[r], kv[r], dot);
-      }
-#pragma unroll
-      for (int offset = kWave / 2; offset >= kPer; offset >>= 1) dot += __shfl_xor(dot, offset, kWave);
-      const float u = beta * (v - dot);
-      float acc = 0.0f;
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const float4 q4 = *(const float4*)(qj + 4 * r4);
-        const float qv[4] = {q4.x, q4.y, q4.z, q4.w};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          S[4 * r4 + i] = fmaf(kv[4 * r4 + i], u, S[4 * r4 + i]);
-          acc = fmaf(S[4 * r4 + i], qv[i], acc);
-        }
-      }
-#pragma unroll
-      for (int offset = kWave / 2; offset >= kPer; offset >>= 1) acc += __shfl_xor(acc, offset, kWave);
-      if (group == 0 && live) a.out[((size_t)(t0 + j) * a.heads + head) * e + col] = acc;
+      for (int r = 0; r < 8; ++r) S[r] = fmaf(kv[r], u, g * S[r]);
+      if (group == 0 && live) a.out[((size_t)(t0 + j) * a.heads + head) * e + col] = fmaf(now.gate.z, u, g * with_q);
     }
   }
   if (!live) return;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = group * 16 + r;
-    if (row < d) state[(size_t)row * e] = S[r];
-  }
+  for (int r = 0; r < 8; ++r)
+    if (group * 8 + r < d) state[r] = S[r];
 }
 
 }  // namespace
 
-// rows [tokens, stride] hold [q | k | v] behind the convolution; ba float32 [tokens, 2 * heads]; out float32 [tokens, heads * value_dim]
+// Floats of scratch that nnis_gated_delta needs for `tokens` rows: the unit vectors, the gates and the products q . k.
+extern "C" long long nnis_gated_delta_scratch(int tokens, int heads, int groups, int key_dim) {
+  return (long long)tokens * ((long long)groups * 2 * key_dim + 2 * heads + groups);
+}
+
+// rows [tokens, stride] hold [q | k | v] behind the convolution; ba float32 [tokens, 2 * heads]; out float32 [tokens, heads *
+// value_dim]; scratch: nnis_gated_delta_scratch floats
 extern "C" int nnis_gated_delta(const void* rows, int dtype, int stride, const float* ba, const float* rate, const float* dt_bias,
                                 float q_scale, float unit_eps, float* state, const int* seq_slot, const int* seq_start, int batch,
-                                int heads, int groups, int key_dim, int value_dim, float* out, void* stream) {
+                                int tokens, int heads, int groups, int key_dim, int value_dim, float* out, float* scratch, void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(dtype), "gated_delta: unknown dtype %d", dtype);
-  NNIS_REQUIRE(heads > 0 && groups > 0 && heads % groups == 0 && key_dim > 0 && key_dim <= 256 && value_dim > 0 && batch >= 0,
+  NNIS_REQUIRE(heads > 0 && groups > 0 && heads % groups == 0 && key_dim > 0 && key_dim <= 256 && value_dim > 0 && batch >= 0 && tokens >= 0,
                "gated_delta: bad sizes (heads %d on %d query/key heads, key channels %d: up to 256 are taken, value channels %d)", heads,
                groups, key_dim, value_dim);
   NNIS_REQUIRE(stride >= 2 * groups * key_dim + heads * value_dim, "gated_delta: rows of %d are too short", stride);
-  NNIS_REQUIRE(rows && ba && rate && dt_bias && state && seq_slot && seq_start && out, "gated_delta: a pointer is missing");
+  NNIS_REQUIRE(rows && ba && rate && dt_bias && state && seq_slot && seq_start && out && scratch, "gated_delta: a pointer is missing");
   NNIS_REQUIRE(batch <= 65535 && heads <= 65535, "gated_delta: %d sequences exceed the grid limit", batch);
-  if (batch == 0) return 0;
+  if (batch == 0 || tokens == 0) return 0;
   DeltaArgs a;
   a.rows = rows; a.dtype = dtype; a.stride = stride; a.ba = ba; a.rate = rate; a.dt_bias = dt_bias; a.q_scale = q_scale;
-  a.unit_eps = unit_eps; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.heads = heads; a.groups = groups;
-  a.key_dim = key_dim; a.value_dim = value_dim; a.out = out;
-  const int need = (key_dim + 15) / 16;
-  const int lane_groups = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : (need <= 8 ? 8 : 16)));
-  const int cols = 4 * (kWave / lane_groups);
-  const int pad = lane_groups * 16;
-  a.chunk = 16;
-  const size_t lds = (size_t)a.chunk * (2 * pad + cols + 2) * sizeof(float);
-  const dim3 grid((value_dim + cols - 1) / cols, heads, batch);
+  a.unit_eps = unit_eps; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.tokens = tokens; a.heads = heads;
+  a.groups = groups; a.key_dim = key_dim; a.value_dim = value_dim; a.out = out;
+  a.unit = scratch;
+  a.gates = scratch + (size_t)tokens * groups * 2 * key_dim;
   hipStream_t s = (hipStream_t)stream;
+  const int items = tokens * groups;
+  hipLaunchKernelGGL(delta_prepare_kernel, dim3((items + 3) / 4), dim3(256), 0, s, a);
+  const int need = (key_dim + 7) / 8;  // a thread keeps 8 key rows
+  const int lane_groups = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : (need <= 8 ? 8 : (need <= 16 ? 16 : 32))));
+  const int cols = 4 * (kWave / lane_groups);
+  const int pad = lane_groups * 8;
+  a.chunk = lane_groups >= 32 ? 16 : 32;  // (kChunk of the kernel)
+  const size_t lds = (size_t)a.chunk * (2 * pad + cols + 4) * sizeof(float);
+  const dim3 grid((value_dim + cols - 1) / cols, heads, batch);
   switch (lane_groups) {
     case 1: hipLaunchKernelGGL(gated_delta_kernel<1>, grid, dim3(256), lds, s, a); break;
     case 2: hipLaunchKernelGGL(gated_delta_kernel<2>, grid, dim3(256), lds, s, a); break;
     case 4: hipLaunchKernelGGL(gated_delta_kernel<4>, grid, dim3(256), lds, s, a); break;
     case 8: hipLaunchKernelGGL(gated_delta_kernel<8>, grid, dim3(256), lds, s, a); break;
-    default: hipLaunchKernelGGL(gated_delta_kernel<16>, grid, dim3(256), lds, s, a); break;
+    case 16: hipLaunchKernelGGL(gated_delta_kernel<16>, grid, dim3(256), lds, s, a); break;
+    default: hipLaunchKernelGGL(gated_delta_kernel<32>, grid, dim3(256), lds, s, a); break;
   }
   NNIS_LAUNCH_CHECK("gated_delta");
   return 0;

@@ -193,6 +193,56 @@ __global__ __launch_bounds__(256) void rms_between_kernel(float* x, const void* 
     store_from_f32(h, h_dtype, base + c, x[base + c] * inv2 * load_as_f32(w_in, w_dtype, c));
 }
 
+// The same, four channels a thread and access (rows of a multiple of four channels, up to 16 x the block's threads):
+// y, the shared rows and the rows out in one type T, the weights in W; the stream, y and both weights are asked for
+// before the first sum is waited for.
+template <typename T, typename W>
+__global__ __launch_bounds__(256) void rms_between4_kernel(float* x, const T* __restrict__ y, const W* __restrict__ w_out,
+                                                           const W* __restrict__ w_in, float eps, T* h, int width,
+                                                           const float* __restrict__ keep, const T* __restrict__ h_in) {
+  __shared__ float scratch[16];
+  __shared__ float scratch2[16];
+  const size_t base = (size_t)blockIdx.x * width;
+  const float share = keep ? keep[blockIdx.x] : 0.0f;
+  float4 ys[kPostKeep4], xs[kPostKeep4], wo[kPostKeep4], wi[kPostKeep4];
+  float ss = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kPostKeep4; ++i) {
+    const int c = 4 * (threadIdx.x + i * blockDim.x);
+    if (c < width) {
+      ys[i] = load4(y + base + c);
+      xs[i] = load4(x + base + c);
+      wo[i] = load4(w_out + c);
+      if (h) wi[i] = load4(w_in + c);
+      if (keep) {
+        const float4 r = load4(h_in + base + c);
+        ys[i].x = fmaf(share, r.x, ys[i].x); ys[i].y = fmaf(share, r.y, ys[i].y);
+        ys[i].z = fmaf(share, r.z, ys[i].z); ys[i].w = fmaf(share, r.w, ys[i].w);
+      }
+      ss = fmaf(ys[i].x, ys[i].x, fmaf(ys[i].y, ys[i].y, fmaf(ys[i].z, ys[i].z, fmaf(ys[i].w, ys[i].w, ss))));
+    }
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  float ss2 = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kPostKeep4; ++i) {
+    const int c = 4 * (threadIdx.x + i * blockDim.x);
+    if (c < width) {
+      xs[i].x += ys[i].x * inv * wo[i].x; xs[i].y += ys[i].y * inv * wo[i].y;
+      xs[i].z += ys[i].z * inv * wo[i].z; xs[i].w += ys[i].w * inv * wo[i].w;
+      store4(x + base + c, xs[i]);
+      ss2 = fmaf(xs[i].x, xs[i].x, fmaf(xs[i].y, xs[i].y, fmaf(xs[i].z, xs[i].z, fmaf(xs[i].w, xs[i].w, ss2))));
+    }
+  }
+  if (h == nullptr) return;
+  const float inv2 = 1.0f / sqrtf(block_sum(ss2, scratch2) / (float)width + eps);
+#pragma unroll
+  for (int i = 0; i < kPostKeep4; ++i) {
+    const int c = 4 * (threadIdx.x + i * blockDim.x);
+    if (c < width) store4(h + base + c, make_float4(xs[i].x * inv2 * wi[i].x, xs[i].y * inv2 * wi[i].y, xs[i].z * inv2 * wi[i].z, xs[i].w * inv2 * wi[i].w));
+  }
+}
+
 // -----------------------------------------------------------------------------
 // PolyNorm: out = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e, powers element by element, each root mean
 // square over the row with eps inside the root; coef = (a, b, c, e) in device memory.
@@ -837,6 +887,22 @@ extern "C" int nnis_rms_between(float* x, const void* y, int y_dtype, const void
   NNIS_REQUIRE((keep == nullptr) == (h_in == nullptr) && (h_in == nullptr || nnis_dtype_ok(h_in_dtype)), "rms_between: a share of rows needs both");
   NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(w_dtype) && (h == nullptr || nnis_dtype_ok(h_dtype)), "rms_between: unknown dtype");
   if (rows <= 0) return 0;
+  // four channels a thread where the types and the row's length allow
+  const int threads4 = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
+  const bool fits4 = width % 4 == 0 && width <= 4 * kPostKeep4 * threads4 && (uintptr_t)y % 16 == 0 && (uintptr_t)x % 16 == 0 &&
+                     (uintptr_t)w_out % 16 == 0 && (uintptr_t)w_in % 16 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)h_in % 16 == 0 &&
+                     (h == nullptr || h_dtype == y_dtype) && (h_in == nullptr || h_in_dtype == y_dtype);
+#define NNIS_BETWEEN4(T_, W_)                                                                                                     \
+  hipLaunchKernelGGL((rms_between4_kernel<T_, W_>), dim3(rows), dim3(threads4), 0, (hipStream_t)stream, x, (const T_*)y, (const W_*)w_out, \
+                     (const W_*)w_in, eps, (T_*)h, width, keep, (const T_*)h_in)
+  if (fits4 && (y_dtype == NNIS_BF16 || w_dtype == NNIS_F32)) {
+    if (y_dtype == NNIS_BF16 && w_dtype == NNIS_BF16) NNIS_BETWEEN4(bf16_t, bf16_t);
+    else if (y_dtype == NNIS_BF16) NNIS_BETWEEN4(bf16_t, float);
+    else NNIS_BETWEEN4(float, float);
+    NNIS_LAUNCH_CHECK("rms_between");
+    return 0;
+  }
+#undef NNIS_BETWEEN4
   hipLaunchKernelGGL(rms_between_kernel, dim3(rows), dim3(width >= 1024 ? 256 : (width >= 256 ? 128 : 64)), 0, (hipStream_t)stream, x, y,
                      y_dtype, w_out, w_in, w_dtype, eps, h, h_dtype, width, keep, h_in, h_in_dtype);
   NNIS_LAUNCH_CHECK("rms_between");

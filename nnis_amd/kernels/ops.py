@@ -103,8 +103,8 @@ _RECURRENT_SIGNATURES = {
                       _VOID, _INT, _INT, _VOID, _VOID, _VOID],
     "nnis_gla_scan_turned": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _VOID, _FLT, _VOID,
                              _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT, _INT, _VOID, _VOID, _VOID],
-    "nnis_gated_delta": [_VOID, _INT, _INT, _VOID, _VOID, _VOID, _FLT, _FLT, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID,
-                         _VOID],
+    "nnis_gated_delta": [_VOID, _INT, _INT, _VOID, _VOID, _VOID, _FLT, _FLT, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _INT, _VOID,
+                         _VOID, _VOID],
     "nnis_gla_decays": [_VOID, _VOID, _INT, _INT, _FLT, _VOID],
     "nnis_head_norm_gate": [_VOID, _VOID, _INT, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _FLT, _VOID],
     "nnis_min_gru": [_VOID, _INT, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT, _INT, _VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID],
@@ -1722,8 +1722,8 @@ def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.T
 
 def gated_delta(rows: torch.Tensor, ba: torch.Tensor, rate: torch.Tensor, dt_bias: torch.Tensor, q_scale: float, state: torch.Tensor,
                 ctx, heads: int, groups: int, key_dim: int, value_dim: int, out: torch.Tensor, unit_eps: float = 1e-6) -> torch.Tensor:
-    """The gated delta rule over each sequence's tokens, from and into ``state`` (float32 [slots, heads, key channels,
-    value channels]): S <- g S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q, raw, float32 [tokens, heads * value
+    """The gated delta rule over each sequence's tokens, from and into ``state`` (float32 [slots, heads, value channels,
+    key channels]: S column by column): S <- g S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q, raw, float32 [tokens, heads * value
     channels].  ``rows`` [tokens, >= 2 * groups * key_dim + heads * value_dim]: q and k of ``groups`` heads, then v; q
     and k are made unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q also times ``q_scale``.  ``ba`` float32
     [tokens, 2 * heads]: beta = sigmoid(first half), g = exp(-rate * softplus(second half + dt_bias)); ``rate`` and
@@ -1737,16 +1737,18 @@ def gated_delta(rows: torch.Tensor, ba: torch.Tensor, rate: torch.Tensor, dt_bia
     for t, what in ((rate, "rate"), (dt_bias, "dt_bias")):
         if t.dtype != torch.float32 or t.numel() != heads:
             raise KernelError(f"gated_delta: {what} must be float32 [{heads}]")
-    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, key_dim, value_dim):
-        raise KernelError(f"gated_delta: state must be float32 [slots, {heads}, {key_dim}, {value_dim}], got {tuple(state.shape)}")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, value_dim, key_dim):
+        raise KernelError(f"gated_delta: state must be float32 [slots, {heads}, {value_dim}, {key_dim}], got {tuple(state.shape)}")
     if out.dtype != torch.float32 or tuple(out.shape) != (tokens, heads * value_dim):
         raise KernelError("gated_delta: out must be float32 [tokens, heads * value channels]")
     _step_arrays(ctx, "gated_delta")
+    # between the two kernels: the unit vectors, g and beta, and the products q . k, all 32-bit
+    scratch = torch.empty(max(1, tokens * (groups * 2 * key_dim + 2 * heads + groups)), dtype=torch.float32, device=out.device)
     lib = recurrent()
     _check(lib, lib.nnis_gated_delta(rows.data_ptr(), _code(rows), rows.stride(0) if tokens > 1 else rows.shape[1], ba.data_ptr(),
                                      rate.data_ptr(), dt_bias.data_ptr(), float(q_scale), float(unit_eps), state.data_ptr(),
-                                     ctx.seq_slot.data_ptr(), ctx.seq_start.data_ptr(), ctx.batch, heads, groups, key_dim, value_dim,
-                                     out.data_ptr(), _stream()))
+                                     ctx.seq_slot.data_ptr(), ctx.seq_start.data_ptr(), ctx.batch, tokens, heads, groups, key_dim,
+                                     value_dim, out.data_ptr(), scratch.data_ptr(), _stream()))
     return out
 
 

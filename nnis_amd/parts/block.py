@@ -215,6 +215,7 @@ class PrePostNormBlock(Block):
         if (feed_forward is None) != (norm2 is None) or (feed_forward is None) != (post2 is None):
             raise InvalidInput("a feed-forward comes with its two norms, or none of the three")
         self.norm1 = build_part("norm", norm1)
+        self.norm1.rows_may_be_prepared = True  # the block before may run this norm in its own last kernel (``PreparedRows``)
         self.post1 = build_part("norm", post1)
         self.mixer = build_part("mixer", mixer, positions=positions)
         self.norm2 = build_part("norm", norm2) if norm2 is not None else None
@@ -267,6 +268,11 @@ class PrePostNormBlock(Block):
                 and post.weight is not None and following.weight is not None and post.weight.dtype == following.weight.dtype)
 
     @classmethod
+    def _hands_rms_rows(cls, post, following) -> bool:
+        """Whether the next block's first norm may be run here: an RMS pair, and a block behind it that takes the rows."""
+        return following is not None and getattr(following, "rows_may_be_prepared", False) and cls._rms_pair(post, following)
+
+    @classmethod
     def _between(cls, x, y, post, following, rt, share=None):
         """x += post(y) in place; returns following(x).  ``share``: (a factor per row, rows): y stands for y + factor * rows."""
         if hasattr(post, "triple") and hasattr(following, "triple") and share is None:
@@ -300,7 +306,7 @@ class PrePostNormBlock(Block):
         share = None
         if self.feed_forward is not None:
             h = y.h if isinstance(y, PreparedRows) else self._between(x, y, self.post1, self.norm2, rt)
-            if getattr(self.feed_forward, "can_leave_share", False) and following is not None and self._rms_pair(self.post2, following):
+            if getattr(self.feed_forward, "can_leave_share", False) and self._hands_rms_rows(self.post2, following):
                 # (a feed-forward that hands a share of its input through leaves that sum to the step's kernel)
                 y = self.feed_forward.forward(h, ctx, rt, share_later=True)
                 y, share = y if isinstance(y, tuple) else (y, None)
@@ -309,7 +315,7 @@ class PrePostNormBlock(Block):
             post = self.post2
         if isinstance(y, PreparedRows):
             return y
-        if following is not None and ((hasattr(post, "triple") and hasattr(following, "triple")) or self._rms_pair(post, following)):
+        if following is not None and ((hasattr(post, "triple") and hasattr(following, "triple")) or self._hands_rms_rows(post, following)):
             return PreparedRows(following, x, self._between(x, y, post, following, rt, share=share))
         return x, PostNormed(y, post)
 

@@ -292,7 +292,8 @@ class GatedDeltaRule(Mixer):
         return small + sum(p.weight_bytes() for p in (self.qkvg, self.ba, self.out))
 
     def cache_request(self):
-        return (StateRequest((self.heads, self.key_dim, self.value_dim)), StateRequest((self.taps - 1, self.channels)))
+        # (the matrix state lies column by column: a value channel's key rows are consecutive)
+        return (StateRequest((self.heads, self.value_dim, self.key_dim)), StateRequest((self.taps - 1, self.channels)))
 
     def forward(self, x, ctx, view, rt):
         state, conv_state = view

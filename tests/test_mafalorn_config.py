@@ -110,7 +110,7 @@ def test_the_cache_it_asks_for():
     keys by the rotated part, in a window's group where it has one."""
     requests, shared = DecoderModel(spec_from_config(MAF_A)[1]).cache_requests()
     assert shared == {}
-    assert requests == [(0, (KVRequest(2, 32, None, None), (StateRequest((4, 16, 24)), StateRequest((2, 2 * 2 * 16 + 4 * 24))))),
+    assert requests == [(0, (KVRequest(2, 32, None, None), (StateRequest((4, 24, 16)), StateRequest((2, 2 * 2 * 16 + 4 * 24))))),
                         (1, StateRequest((3, 16, 32))), (2, KVRequest(1, 48, 37, 40)), (3, StateRequest((2, 24, 8)))]
     requests, _ = DecoderModel(spec_from_config(MAF_C)[1]).cache_requests()
     assert dict(requests)[1] == KVRequest(1, 32, None, 24)

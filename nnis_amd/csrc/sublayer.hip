@@ -484,7 +484,7 @@ __device__ __forceinline__ void router_dots(const float* xs, const float* __rest
 // Logits and choice in one kernel: a block takes R rows (as floats in LDS), its waves the outputs' dot products into
 // LDS, then wave r routes row r.
 template <int R>
-__global__ __launch_bounds__(256) void route_kernel(const void* __restrict__ x, int x_dtype, const float* __restrict__ w,
+__global__ __launch_bounds__(R == 1 ? 1024 : 256) void route_kernel(const void* __restrict__ x, int x_dtype, const float* __restrict__ w,
                                                     const float* __restrict__ correction, int rows, int n, int width, int experts,
                                                     int top, float* __restrict__ gates, float* __restrict__ keep, int group_count,
                                                     int group_keep) {
@@ -972,7 +972,9 @@ extern "C" int nnis_route(const void* x, int x_dtype, const float* w, const floa
     hipLaunchKernelGGL((route_kernel<2>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep,
                        group_count, group_keep);
   } else {
-    hipLaunchKernelGGL((route_kernel<1>), grid, dim3(256), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep,
+    // a row a block: a wave an output where the outputs are many, so that every weight row is asked for at once
+    const int threads = n > 8 ? 1024 : (n > 4 ? 512 : 256);
+    hipLaunchKernelGGL((route_kernel<1>), grid, dim3(threads), lds, s, x, x_dtype, w, correction, rows, n, width, experts, top, gates, keep,
                        group_count, group_keep);
   }
   NNIS_LAUNCH_CHECK("route");

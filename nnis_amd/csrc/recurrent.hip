@@ -986,12 +986,14 @@ __device__ __forceinline__ DeltaToken delta_token(const float* qk, const float* 
                                                   int cols) {
   constexpr int kPad = GROUPS * 8;
   DeltaToken t;
-  const float* qj = qk + j * 2 * kPad + group * 8;
+  // (a thread's 8 key rows are two runs of 4, half the padded rows apart: a column's lanes then read 16 bytes each of
+  // consecutive LDS, and no two of them meet in a bank)
+  const float* qj = qk + j * 2 * kPad + group * 4;
   const float* kj = qj + kPad;
   t.k[0] = *(const float4*)kj;
-  t.k[1] = *(const float4*)(kj + 4);
+  t.k[1] = *(const float4*)(kj + kPad / 2);
   t.q[0] = *(const float4*)qj;
-  t.q[1] = *(const float4*)(qj + 4);
+  t.q[1] = *(const float4*)(qj + kPad / 2);
   t.gate = *(const float4*)(gs + 4 * j);
   t.v = vs[j * cols + col_in_block];
   return t;
@@ -1017,25 +1019,30 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(DeltaArgs a) {
   const int d = a.key_dim, e = a.value_dim;
   const int qk_head = head / (a.heads / a.groups);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int group = lane % GROUPS;             // which 8 key rows
+  const int group = lane % GROUPS;             // which 8 key rows (two runs of 4)
   const int col_in_block = wave * kPer + lane / GROUPS;
   const int col = blockIdx.x * kCols + col_in_block;
   const bool live = col < e;
   float* qk = lds;                        // [chunk][2][kPad]: a token's q, then its k
   float* vs = qk + kChunk * 2 * kPad;     // [chunk][kCols]
   float* gs = vs + kChunk * kCols;        // [chunk][4]: g, beta, q . k
-  float* state = a.state + (((size_t)slot * a.heads + head) * e + (live ? col : 0)) * d + group * 8;
+  float* state = a.state + (((size_t)slot * a.heads + head) * e + (live ? col : 0)) * d;
+  int rows[8];  // the key rows this thread keeps
+#pragma unroll
+  for (int r = 0; r < 8; ++r) rows[r] = (r < 4 ? 0 : kPad / 2) + group * 4 + r % 4;
   float S[8];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) S[r] = live && group * 8 + r < d ? state[r] : 0.0f;
+  for (int r = 0; r < 8; ++r) S[r] = live && rows[r] < d ? state[rows[r]] : 0.0f;
   const size_t v_col0 = 2 * (size_t)a.groups * d;
   const float* qk_dots = a.gates + (size_t)a.tokens * a.heads * 2;
   const bool whole = d == kPad;  // a token's q and k are what LDS holds of it: copied 16 bytes at a time
-  for (int t0 = begin; t0 < end; t0 += kChunk) {
+  // A chunk's numbers wait in registers while the chunk before is worked on: they are asked for from memory before
+  // that work begins, so a chunk's loads cost the recurrence nothing but the registers.
+  float4 qk_in[kQkLoads];
+  float v_in[kVLoads];
+  float gate_in[3] = {0.0f, 0.0f, 0.0f};
+  auto ask = [&](int t0) {
     const int count = min(kChunk, end - t0);
-    float4 qk_in[kQkLoads];
-    float v_in[kVLoads];
-    float gate_in[3] = {0.0f, 0.0f, 0.0f};
     if (whole) {
 #pragma unroll
       for (int it = 0; it < kQkLoads; ++it) {
@@ -1055,6 +1062,10 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(DeltaArgs a) {
       gate_in[1] = a.gates[2 * ((size_t)t * a.heads + head) + 1];
       gate_in[2] = qk_dots[(size_t)t * a.groups + qk_head];
     }
+  };
+  ask(begin);
+  for (int t0 = begin; t0 < end; t0 += kChunk) {
+    const int count = min(kChunk, end - t0);
     __syncthreads();  // the chunk before has been read
     if (whole) {
 #pragma unroll
@@ -1079,11 +1090,13 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(DeltaArgs a) {
       gs[4 * threadIdx.x + 2] = gate_in[2];
     }
     __syncthreads();
+    if (t0 + kChunk < end) ask(t0 + kChunk);  // the next chunk's numbers, in flight from here on
     // a token's numbers are read from LDS while the token before is worked on
     DeltaToken next = delta_token<GROUPS>(qk, vs, gs, 0, group, col_in_block, kCols);
     for (int j = 0; j < count; ++j) {
       const DeltaToken now = next;
       if (j + 1 < count) next = delta_token<GROUPS>(qk, vs, gs, j + 1, group, col_in_block, kCols);
+      __builtin_amdgcn_sched_barrier(0);  // (the reads stay up here, ahead of the work on the token before: left to itself the compiler moves them down to their use)
       const float kv[8] = {now.k[0].x, now.k[0].y, now.k[0].z, now.k[0].w, now.k[1].x, now.k[1].y, now.k[1].z, now.k[1].w};
       const float qv[8] = {now.q[0].x, now.q[0].y, now.q[0].z, now.q[0].w, now.q[1].x, now.q[1].y, now.q[1].z, now.q[1].w};
       float dot_k[2] = {0.0f, 0.0f}, dot_q[2] = {0.0f, 0.0f};
@@ -1106,7 +1119,7 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(DeltaArgs a) {
   if (!live) return;
 #pragma unroll
   for (int r = 0; r < 8; ++r)
-    if (group * 8 + r < d) state[r] = S[r];
+    if (rows[r] < d) state[rows[r]] = S[r];
 }
 
 }  // namespace

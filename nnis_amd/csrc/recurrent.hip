@@ -1,6 +1,8 @@
 // Mixers that carry a state of fixed size from token to token: a short causal convolution per channel, the
 // selective scan (a diagonal recurrence per channel with input-dependent steps), gated linear attention (a
-// matrix state per head with a decay per key channel), and the per-head norm and gate behind it.
+// matrix state per head with a decay per key channel; with one fixed decay a head and turned queries and keys it
+// is retention), the per-head norm and gate behind it, the minGRU, and the gated delta rule (a matrix state per
+// head whose every token first takes back what the state already holds under its key).
 //
 // A step's rows are packed: sequence b of the step owns rows seq_start[b] .. seq_start[b + 1] - 1, which
 // continue the sequence in slot seq_slot[b] (negative: padding, nothing is read or written for it).  State

@@ -146,7 +146,7 @@ def _attention_recipe(rest: str) -> ModuleRecipe:
 register_module("core", ["elementwise.hip", "residual.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"],
                 headers=["common.h", "epilogue.h", "nnis_noalloc.h"], source_flags={"gemm_mfma.hip": _VECTOR_SUMS})
 register_module_family("attn_hd", _attention_recipe)
-# the mixers that carry a state of fixed size (convolution, selective scan, gated linear attention)
+# the mixers that carry a state of fixed size (convolution, selective scan, gated linear attention and retention, minGRU, gated delta rule)
 register_module("recurrent", ["recurrent.hip"], headers=["common.h"])
 # attention over a cached latent: what lies between its projections (norms of the latents, rotation, cache write, gates)
 register_module("latent", ["latent.hip"], headers=["common.h"])

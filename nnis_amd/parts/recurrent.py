@@ -246,7 +246,7 @@ class GatedDeltaRule(Mixer):
         S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q                   per head, S [d, e]
         out = W_o (concat_h(o / rms(o) * w_norm) * silu(W_g h))
 
-    State per sequence: S [H, d, e] and the convolution's last ``taps`` - 1 inputs.  Queries, keys, values and the gate
+    State per sequence: S, kept column by column as [H, e, d], and the convolution's last ``taps`` - 1 inputs.  Queries, keys, values and the gate
     leave one projection and one convolution; beta's and the decay's logits leave a second projection in 32-bit; unit
     vectors, beta, decays, the recurrence and the norm are 32-bit under either runtime."""
 
